@@ -99,14 +99,19 @@ class KernelBackend:
             return self.linear_silu_mul(x, w_gate_up, intermediate)
         raise NotImplementedError
 
+    def linear_act(self, x, w, activation="relu2"):
+        """act(x w^T), act one of ACTIVATIONS, computed on the product's 32-bit sums and rounded once
+        -> [T, out] in the activation dtype.  ``x`` is a tensor or a Normed."""
+        raise NotImplementedError
+
     def scale_(self, t, factor):
         """t *= factor in place (float32), returns t."""
         raise NotImplementedError
 
-    def branch_norm_add(self, y, stream, weight, eps):
+    def branch_norm_add(self, y, stream, weight, eps, copy=True):
         """stream += y * rsqrt(mean(y^2) + eps) * weight, row by row in float32 (y [T, width] of any float
         dtype; None: nothing is added).  Returns the updated stream in the activation dtype, rounded once
-        (the stream itself where that is float32)."""
+        (the stream itself where that is float32); with ``copy`` False nothing is returned (and no copy made)."""
         raise NotImplementedError
 
     def rmsnorm_columns(self, x, col, n, weight, eps):
@@ -159,14 +164,21 @@ class KernelBackend:
         raise NotImplementedError
 
     # ---- routed experts
-    def route_topk(self, logits, bias, top):
-        """logits [T, E] float32 (+ bias [E]): the ``top`` largest of a token (lowest index first among equals), in
-        falling order, and the softmax over those alone -> (experts [T, top] int32, shares [T, top] float32)."""
+    def route_topk(self, logits, bias, top, over="chosen", choice_bias=None):
+        """logits [T, E] float32 (+ bias [E]).  ``over`` "chosen": the ``top`` largest of a token (lowest index first
+        among equals), in falling order, and the softmax over those alone.  ``over`` "all": scores = softmax over all
+        E; chosen are the ``top`` largest of scores + choice_bias (float32 [E] or None; lowest index first among
+        equals, falling order) and the shares are the chosen ones' scores as they are, not renormalised.
+        -> (experts [T, top] int32, shares [T, top] float32)."""
         raise NotImplementedError
 
-    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2"):
+    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None):
         """y[t] = sum_j shares[t, j] * W_down[e] act(W_up[e] x[t]), e = experts[t, j]; w_up [E, ff, width],
-        w_down [E, width, ff]; the hidden activation is rounded once to the activation dtype -> [T, width] float32."""
+        w_down [E, width, ff]; the hidden activation is rounded once to the activation dtype -> [T, width] float32.
+        ``gated`` = (limit, alpha): w_up is [E, 2 ff, width], an expert's gate rows before its up rows, and the hidden
+        activation is g * sigmoid(alpha g) * (u + 1) with g = min(gate sum, limit), u = clamp(up sum, -limit, limit),
+        ``activation`` unused.  ``identity_from`` = E: a choice e >= E is an expert that returns x[t] itself (such
+        choices may be all there are: w_up and w_down None)."""
         raise NotImplementedError
 
     # ---- a short convolution on a mixer's input, attention from one product's sums, the delta rule
@@ -187,11 +199,14 @@ class KernelBackend:
         return x, (None if w_second is None else self.add_rmsnorm(None, stream, w_second, eps))
 
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
-                   layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None):
+                   layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None,
+                   norm_per_head=False):
         """What lies between a q/k/v projection's float32 sums [T, *] and attention, in 32-bit: queries are columns
         [q_col, q_col + Hq dim), keys [k_col, k_col + Hkv dim), values [v_col, v_col + Hkv vdim), or, with ``v_col``
         None, the keys as projected (vdim = dim).  ``q_norm`` / ``k_norm`` (float32 [Hq dim] / [Hkv dim]): RMS norm over
-        the whole of a token's queries (keys) at once, times that weight, before anything else.  Then the first
+        the whole of a token's queries (keys) at once, times that weight, before anything else; with ``norm_per_head`` the
+        norm is taken head by head over the head's dim numbers and the weights are float32 [dim], one for all query
+        heads and one for all key heads.  Then the first
         2 * len(inv_freq) numbers of every query and key head turn by the angles position * inv_freq[i]: ``layout``
         "interleaved" pairs (2i, 2i + 1), "half" pairs (i, i + len(inv_freq)).  ``q_head_scale`` (float32 [Hq]):
         head h's turned query times that number.  Keys and values go to the token's slot of k_cache [pages, Hkv, page, P]
@@ -243,12 +258,15 @@ class KernelBackend:
         return qkv
 
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
-                        window, sink=None):
+                        window, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None):
         """For token t of row r at position p: softmax over keys max(0, p - window + 1)..p
         of row r (read through group.block_tables[r]) of (q . k) * scale, times v.
         q head i uses kv head i // (Hq / Hkv).  q is the first Hq * D columns of
         qkv (row stride qkv.stride(0)).  ``sink`` (a number): one more term exp(sink) in every softmax's
-        denominator, with no value.  Returns [T, Hq * D] in act_dtype."""
+        denominator, with no value.  ``chunk`` (a number of positions): keys before floor(p / chunk) * chunk are not
+        seen either.  ``softcap`` (c > 0): the scaled scores pass through c * tanh(score / c).  ``weights`` "sigmoid":
+        no softmax; a visible key counts with sigmoid(score + head_bias[i]) (head_bias float32 [Hq] or None), not
+        normalised over the keys (no sink).  Returns [T, Hq * D] in act_dtype."""
         raise NotImplementedError
 
     def sample(self, logits, temperatures, seeds, counters, out=None):

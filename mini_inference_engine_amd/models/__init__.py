@@ -1,7 +1,9 @@
 from . import llama  # noqa: F401  (registers LlamaForCausalLM)
 from . import zifelorn  # noqa: F401  (registers Zifelorn)
 from . import vezodra  # noqa: F401  (registers Vezodra)
+from . import mutusun  # noqa: F401  (registers Mutusun)
 from .decoder import Decoder
 from .llama import build_llama
 from .zifelorn import build_zifelorn
 from .vezodra import build_vezodra
+from .mutusun import build_mutusun

@@ -141,3 +141,62 @@ class ParallelBlock(Block):
             if f is not None:
                 residual.add_(f.float())
         return None, residual
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """A norm before and after each sublayer, and an optional short convolution on what each sublayer reads:
+    stream += norm_mixer_out(mixer(c1(norm_mixer(stream)))); stream += norm_feed_forward_out(feed_forward(c2(
+    norm_feed_forward(stream)))).  ``conv_mixer`` / ``conv_feed_forward`` (c1, c2: parts.ResidualConv or None) keep
+    their last inputs beside the mixer's cache (CombinedCache members ``mixer``, ``conv1``, ``conv2``).  The
+    feed-forward (with its two norms and its convolution) may be None.  Norms, convolutions and adds are 32-bit;
+    the sublayers hand their 32-bit sums to the norm after them."""
+
+    def __init__(self, norm_mixer, mixer, norm_mixer_out, norm_feed_forward=None, feed_forward=None,
+                 norm_feed_forward_out=None, conv_mixer=None, conv_feed_forward=None):
+        if len({feed_forward is None, norm_feed_forward is None, norm_feed_forward_out is None}) != 1:
+            raise ValueError("a feed-forward and its two norms come together or not at all")
+        if feed_forward is None and conv_feed_forward is not None:
+            raise ValueError("a convolution on the feed-forward's input needs a feed-forward")
+        self.norm_mixer, self.mixer, self.norm_mixer_out = norm_mixer, mixer, norm_mixer_out
+        self.norm_feed_forward, self.feed_forward = norm_feed_forward, feed_forward
+        self.norm_feed_forward_out = norm_feed_forward_out
+        self.conv_mixer, self.conv_feed_forward = conv_mixer, conv_feed_forward
+
+    def children(self):
+        return [p for p in (self.norm_mixer, self.conv_mixer, self.mixer, self.norm_mixer_out, self.norm_feed_forward,
+                            self.conv_feed_forward, self.feed_forward, self.norm_feed_forward_out) if p is not None]
+
+    def cache_requirement(self):
+        if self.conv_mixer is None and self.conv_feed_forward is None:
+            return self.mixer.cache_requirement()
+        return CombinedCache([("mixer", self.mixer.cache_requirement()),
+                              ("conv1", None if self.conv_mixer is None else self.conv_mixer.cache_requirement()),
+                              ("conv2", None if self.conv_feed_forward is None else self.conv_feed_forward.cache_requirement())])
+
+    def _read(self, residual, norm, conv, cache, member, step):
+        """What a sublayer reads: the normed stream, through its convolution if it has one."""
+        import torch
+        ops = self.ops
+        if conv is None:
+            return ops.add_rmsnorm(None, residual, norm.weight, norm.eps)
+        w = norm.weight if norm.weight.dtype == torch.float32 else norm.weight.float()
+        return ops.norm_pair_conv(residual, w, None, norm.eps, conv.weight, cache.sub(member).tensors["tail"], step)[0]
+
+    def forward(self, h, residual, step, cache, next_norm=None):
+        ops = self.ops
+        if isinstance(h, Normed):               # a block of another kind before this one: its last add may be pending
+            h = h.pending
+        elif isinstance(h, StreamCopy):
+            h = None
+        if h is not None:
+            residual.add_(h.float())
+        combined = self.conv_mixer is not None or self.conv_feed_forward is not None
+        x = self._read(residual, self.norm_mixer, self.conv_mixer, cache, "conv1", step)
+        a = self.mixer.forward(x, step, cache.sub("mixer") if combined else cache)
+        ops.branch_norm_add(a, residual, self.norm_mixer_out.weight, self.norm_mixer_out.eps, copy=False)
+        if self.feed_forward is not None:
+            y = self._read(residual, self.norm_feed_forward, self.conv_feed_forward, cache, "conv2", step)
+            f = self.feed_forward.forward(y, step)
+            ops.branch_norm_add(f, residual, self.norm_feed_forward_out.weight, self.norm_feed_forward_out.eps, copy=False)
+        return None, residual

@@ -2,8 +2,9 @@
 
 y = weight * x * rsqrt(mean(x^2) + eps), taken of the stream after the pending
 branch output has been added to it (inference_engine/kernels/rmsnorm.py:56-65;
-used at inference_engine/model.py:171,179,184).  The weight is a plain multiplier.
-The stream and every intermediate are 32-bit; y is rounded once.
+used at inference_engine/model.py:171,179,184).  The weight is a plain multiplier, or, with
+``one_plus``, stored around zero and applied as 1 + weight (the sum is made once, in 32-bit, when
+the weights are loaded).  The stream and every intermediate are 32-bit; y is rounded once.
 """
 from __future__ import annotations
 
@@ -13,14 +14,21 @@ from .base import Norm, ParamSpec, register_norm
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
-    def __init__(self, width: int, eps: float, weight_name: str):
+    def __init__(self, width: int, eps: float, weight_name: str, one_plus: bool = False):
         self.width = int(width)
         self.eps = float(eps)
         self.weight_name = weight_name
+        self.one_plus = bool(one_plus)
         self.weight = None
+        self._summed = False
 
     def params(self):
-        return [ParamSpec.single("weight", self.weight_name, (self.width,), init="scale")]
+        return [ParamSpec.single("weight", self.weight_name, (self.width,), init="weight" if self.one_plus else "scale")]
+
+    def prepare(self, device, dtype):
+        if self.one_plus and not self._summed:
+            self._summed = True
+            self.weight = (1.0 + self.weight.float()).contiguous()
 
     def lazy(self, x, residual, rows=None):
         if isinstance(x, Normed):

@@ -125,20 +125,34 @@ def ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tai
     return out.to(out_dtype)
 
 
-def ref_route_topk(logits, bias, top):
+def ref_route_topk(logits, bias, top, over="chosen", choice_bias=None):
     z = logits.double() if bias is None else logits.double() + bias.double()
+    if over == "all":
+        scores = torch.softmax(z.float(), -1).double()
+        by = scores if choice_bias is None else (scores.float() + choice_bias.float()).double()
+        idx = torch.sort(by, dim=-1, descending=True, stable=True).indices[:, :top]
+        return idx.to(torch.int32), torch.gather(scores, 1, idx).float()
     order = torch.sort(z, dim=-1, descending=True, stable=True)
     idx, val = order.indices[:, :top], order.values[:, :top]
     return idx.to(torch.int32), torch.softmax(val, -1).float()
 
 
-def ref_routed_experts(x, experts, shares, w_up, w_down, activation, act_dtype):
-    y = torch.zeros(x.shape[0], w_down.shape[1], dtype=torch.float64, device=x.device)
+def ref_clamped_glu(gu, inner, limit, alpha):
+    g, u = gu[..., :inner].clamp(max=limit), gu[..., inner:].clamp(min=-limit, max=limit)
+    return g * torch.sigmoid(alpha * g) * (u + 1.0)
+
+
+def ref_routed_experts(x, experts, shares, w_up, w_down, activation, act_dtype, gated=None, identity_from=None):
+    y = torch.zeros(x.shape[0], x.shape[1], dtype=torch.float64, device=x.device)
     for t in range(x.shape[0]):
         for j in range(experts.shape[1]):
             e = int(experts[t, j])
-            h = ref_act(x[t].double() @ w_up[e].double().T, activation).to(act_dtype).double()
-            y[t] += shares[t, j].double() * (h @ w_down[e].double().T)
+            if identity_from is not None and e >= identity_from:
+                y[t] += shares[t, j].double() * x[t].double()
+                continue
+            z = x[t].double() @ w_up[e].double().T
+            h = ref_act(z, activation) if gated is None else ref_clamped_glu(z, z.shape[-1] // 2, gated[0], gated[1])
+            y[t] += shares[t, j].double() * (h.to(act_dtype).double() @ w_down[e].double().T)
     return y.float()
 
 
@@ -186,7 +200,7 @@ def ref_rotary_kv_store(qkv, positions, cos, sin, rotary_dim, Hq, Hkv, D, k_cach
 
 
 def ref_paged_attention(qkv, Hq, Hkv, D, k_cache, v_cache, block_tables, token_row, positions, scale, window,
-                        out_dtype, sink=None):
+                        out_dtype, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None):
     """Token by token, keys gathered through the block table."""
     T = qkv.shape[0]
     P = k_cache.shape[2]
@@ -198,13 +212,19 @@ def ref_paged_attention(qkv, Hq, Hkv, D, k_cache, v_cache, block_tables, token_r
     for t in range(T):
         p = pos[t]
         lo = 0 if window is None else max(0, p - window + 1)
+        if chunk is not None:
+            lo = max(lo, p // chunk * chunk)
         keys = torch.arange(lo, p + 1, device=qkv.device)
         pages = bt[rows[t], keys // P]
         k = k_cache[pages, :, keys % P, :].double()          # [n, Hkv, D]
         v = v_cache[pages, :, :, keys % P].double()             # [n, Hkv, D]
         q = qkv[t, :Hq * D].double().view(Hkv, g, D)
         s = torch.einsum("hgd,nhd->hgn", q, k) * scale
-        if sink is None:
+        if softcap is not None:
+            s = softcap * torch.tanh(s / softcap)
+        if weights == "sigmoid":
+            pr = torch.sigmoid(s if head_bias is None else s + head_bias.double().view(Hkv, g, 1))
+        elif sink is None:
             pr = torch.softmax(s, dim=-1)
         else:               # one more term in the denominator, with no value
             top = s.max(-1, keepdim=True).values.clamp(min=sink)
@@ -245,17 +265,19 @@ def ref_turn(x, positions, inv_freq, layout):
 
 
 def ref_qkv_finish(sums, q_col, k_col, v_col, Hq, Hkv, dim, vdim, P, positions, inv_freq, layout, k_cache, v_cache, slots,
-                   q_norm, k_norm, eps, q_head_scale, out_dtype):
+                   q_norm, k_norm, eps, q_head_scale, out_dtype, norm_per_head=False):
     T = sums.shape[0]
     q = sums[:, q_col:q_col + Hq * dim].double()
     k = sums[:, k_col:k_col + Hkv * dim].double()
     v = k if v_col is None else sums[:, v_col:v_col + Hkv * vdim].double()
     v = v.view(T, Hkv, -1)
+    if norm_per_head:
+        q, k = q.view(T, Hq, dim), k.view(T, Hkv, dim)
     if q_norm is not None:
         q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm.double()
     if k_norm is not None:
         k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm.double()
-    q, k = q.view(T, Hq, dim), k.view(T, Hkv, dim)
+    q, k = q.reshape(T, Hq, dim), k.reshape(T, Hkv, dim)
     if inv_freq is not None:
         q, k = ref_turn(q, positions, inv_freq, layout), ref_turn(k, positions, inv_freq, layout)
     if q_head_scale is not None:
@@ -361,7 +383,13 @@ class TorchBackend(KernelBackend):
     def scale_(self, t, factor):
         return t.mul_(factor)
 
-    def branch_norm_add(self, y, stream, weight, eps):
+    def linear_act(self, x, w, activation="relu2"):
+        self._count("linear_act")
+        if isinstance(x, Normed):
+            x = x.materialize()
+        return ref_act(ref_linear(x, w, None, torch.float32).double(), activation).to(self.act_dtype)
+
+    def branch_norm_add(self, y, stream, weight, eps, copy=True):
         self._count("branch_norm_add")
         return ref_branch_norm_add(y, stream, weight, eps, self.act_dtype)
 
@@ -401,12 +429,12 @@ class TorchBackend(KernelBackend):
         return ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step.host["row_start"],
                               step.host["state_slots"], taps, decay_scale, self.act_dtype)
 
-    def route_topk(self, logits, bias, top):
-        return ref_route_topk(logits, bias, top)
+    def route_topk(self, logits, bias, top, over="chosen", choice_bias=None):
+        return ref_route_topk(logits, bias, top, over, choice_bias)
 
-    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2"):
+    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None):
         self._count("routed_experts")
-        return ref_routed_experts(x, experts, shares, w_up, w_down, activation, self.act_dtype)
+        return ref_routed_experts(x, experts, shares, w_up, w_down, activation, self.act_dtype, gated, identity_from)
 
     def add_rmsnorm(self, x, residual, weight, eps, out_dtype=None, rows=None):
         self._count("add_rmsnorm")
@@ -438,20 +466,23 @@ class TorchBackend(KernelBackend):
                             k_cache, v_cache, slot_mapping)
 
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
-                        window, sink=None):
+                        window, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None):
         self._count("paged_attention")
         return ref_paged_attention(qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group.block_tables,
-                                   step.token_row, step.positions, scale, window, self.act_dtype, sink=sink)
+                                   step.token_row, step.positions, scale, window, self.act_dtype, sink=sink,
+                                   weights=weights, softcap=softcap, chunk=chunk, head_bias=head_bias)
 
     def residual_conv(self, h, taps, tail, step, out_dtype=None):
         self._count("residual_conv")
         return ref_residual_conv(h, taps, tail, step.host["row_start"], step.host["state_slots"], out_dtype or self.act_dtype)
 
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
-                   layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None):
+                   layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None,
+                   norm_per_head=False):
         self._count("qkv_finish")
         return ref_qkv_finish(sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
-                              layout, k_cache, v_cache, slot_mapping, q_norm, k_norm, eps, q_head_scale, self.act_dtype)
+                              layout, k_cache, v_cache, slot_mapping, q_norm, k_norm, eps, q_head_scale, self.act_dtype,
+                              norm_per_head)
 
     def head_gate_(self, o, gate, gate_col, num_heads, head_dim):
         o.copy_(ref_head_gate(o, gate, gate_col, num_heads, head_dim))
