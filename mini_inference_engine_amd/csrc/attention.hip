@@ -2,14 +2,17 @@
 // portions starting anywhere), in true 32-bit arithmetic for float and bfloat16 storage.
 //
 // One wavefront per (token, query head).  The token sits in row r at absolute position p and
-// sees keys lo..p of its own request, lo = max(0, p - window + 1) or 0, found through the
+// sees keys lo..p of its own request, lo = max(0, p - window + 1) or 0 (with a chunk size c
+// also lo >= floor(p / c) * c: a query sees its own chunk of positions only), found through the
 // row's block table in caches laid out [pages, Hkv, page, D] (keys) and [pages, Hkv, D, page]
 // (values, transposed within a page).  Keys are taken 64 at a time
 // (one per lane: q . k in increasing d), the softmax is kept online in 32-bit, and the 64
 // probabilities then weight the value rows with the lanes spread over D.  The order of every
 // sum depends only on (lo, p): the result for a token is bit-identical whatever else the
 // step holds and however the request was cut into steps.  With a sink, one more term exp(sink)
-// joins the softmax's denominator at the end and has no value.
+// joins the softmax's denominator at the end and has no value.  With a cap c the scaled scores
+// pass through c * tanh(score / c).  In the sigmoid mode there is no softmax: a visible key counts
+// with sigmoid(score + the head's bias), and the weights are not normalised.
 //
 // This is the reference kernel of the engine: the float32 path runs on it, and the
 // bfloat16 path uses it wherever a faster kernel does not take the shape.
@@ -41,14 +44,17 @@ __global__ void __launch_bounds__(64)
 paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache,
                        const T* __restrict__ v_cache, T* __restrict__ out, const int* __restrict__ block_tables,
                        int max_blocks, const int* __restrict__ token_row, const int* __restrict__ positions, int Hq,
-                       int Hkv, int D, int page, float scale, int window, int has_sink, float sink) {
+                       int Hkv, int D, int page, float scale, int window, int has_sink, float sink, int chunk,
+                       float softcap, int sigmoid, const float* __restrict__ head_bias) {
   __shared__ float qs[NR * 64];
   __shared__ float ps[64];
   __shared__ long long base[64];     // per key of the chunk: offset of its value column
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int row = token_row[t], pos = positions[t];
   const int kvh = h / (Hq / Hkv);
-  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  if (chunk > 0 && pos / chunk * chunk > lo) lo = pos / chunk * chunk;
+  const float hb = sigmoid && head_bias ? head_bias[h] : 0.f;
   const int* bt = block_tables + (size_t)row * max_blocks;
   const T* qp = q + (size_t)t * q_stride + (size_t)h * D;
   for (int d = lane; d < D; d += 64) qs[d] = to_float(qp[d]);
@@ -77,11 +83,18 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
         for (int e = 0; e < P::N; ++e) dot = fmaf(qs[d0 + e], f[e], dot);
       }
       s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
-    const float m_new = fmaxf(m, wave_max(s));      // finite: key c0 <= pos is valid
-    const float alpha = expf(m - m_new);            // 0 on the first chunk (m = -inf)
-    const float p = valid ? expf(s - m_new) : 0.f;
-    l = l * alpha + wave_sum(p);
+    float alpha = 1.f, p;
+    if (sigmoid) {
+      p = valid ? mie_sigmoid(s + hb) : 0.f;
+    } else {
+      const float m_new = fmaxf(m, wave_max(s));    // finite: key c0 <= pos is valid
+      alpha = expf(m - m_new);                      // 0 on the first chunk (m = -inf)
+      p = valid ? expf(s - m_new) : 0.f;
+      l = l * alpha + wave_sum(p);
+      m = m_new;
+    }
     ps[lane] = p;
     __syncthreads();
     const int nk = pos - c0 + 1 < 64 ? pos - c0 + 1 : 64;
@@ -97,16 +110,15 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
       }
     }
     __syncthreads();
-    m = m_new;
   }
-  if (has_sink) {                     // one more term exp(sink) in the denominator, with no value
+  if (has_sink && !sigmoid) {                     // one more term exp(sink) in the denominator, with no value
     const float m_new = fmaxf(m, sink);
     const float alpha = expf(m - m_new);
     l = l * alpha + expf(sink - m_new);
 #pragma unroll
     for (int i = 0; i < NR; ++i) acc[i] *= alpha;
   }
-  const float inv = 1.0f / l;
+  const float inv = sigmoid ? 1.0f : 1.0f / l;
   T* op = out + ((size_t)t * Hq + h) * D;
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
@@ -117,11 +129,14 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
 
 MIE_EXPORT const char* attention_last_error() { return g_mie_error; }
 
-MIE_EXPORT int mie_paged_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+static int paged_attention_launch(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
                                    int dtype, const int* block_tables, int max_blocks, const int* token_row,
                                    const int* positions, int tokens, int Hq, int Hkv, int D, int page, float scale,
-                                   int window, int has_sink, float sink, hipStream_t stream) {
+                                   int window, int has_sink, float sink, int chunk, float softcap, int sigmoid,
+                                   const float* head_bias, hipStream_t stream) {
   if (tokens <= 0) return 0;
+  if (chunk < 0 || softcap < 0.f) MIE_FAIL("paged_attention: chunk %d, score cap %g", chunk, (double)softcap);
+  if (sigmoid && has_sink) MIE_FAIL("paged_attention: a sink belongs to a softmax; the weights asked for are sigmoids");
   if (D % 16 || D < 16 || D > ATT_MAX_D) MIE_FAIL("paged_attention: head_dim %d (multiples of 16 up to %d)", D, ATT_MAX_D);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("paged_attention: %d query heads on %d kv heads", Hq, Hkv);
   if (Hq > 65535) MIE_FAIL("paged_attention: %d query heads is beyond the grid", Hq);
@@ -131,7 +146,7 @@ MIE_EXPORT int mie_paged_attention(const void* q, long q_stride, const void* k_c
 #define PA_LAUNCH(T_, NR_)                                                                                               \
   hipLaunchKernelGGL((paged_attention_kernel<T_, NR_>), grid, block, 0, stream, (const T_*)q, q_stride, (const T_*)k_cache, \
                      (const T_*)v_cache, (T_*)out, block_tables, max_blocks, token_row, positions, Hq, Hkv, D, page, scale,  \
-                     window, has_sink, sink)
+                     window, has_sink, sink, chunk, softcap, sigmoid, head_bias)
   if (dtype == MIE_F32 && D <= 256) PA_LAUNCH(float, 4);
   else if (dtype == MIE_F32) PA_LAUNCH(float, 16);
   else if (dtype == MIE_BF16 && D <= 256) PA_LAUNCH(bf16, 4);
@@ -140,4 +155,24 @@ MIE_EXPORT int mie_paged_attention(const void* q, long q_stride, const void* k_c
 #undef PA_LAUNCH
   MIE_CHECK_LAUNCH("paged_attention");
   return 0;
+}
+
+MIE_EXPORT int mie_paged_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                   int dtype, const int* block_tables, int max_blocks, const int* token_row,
+                                   const int* positions, int tokens, int Hq, int Hkv, int D, int page, float scale,
+                                   int window, int has_sink, float sink, hipStream_t stream) {
+  return paged_attention_launch(q, q_stride, k_cache, v_cache, out, dtype, block_tables, max_blocks, token_row, positions,
+                                tokens, Hq, Hkv, D, page, scale, window, has_sink, sink, 0, 0.f, 0, nullptr, stream);
+}
+
+// The same with what a design may put between scores and weights: a chunk size (0: none), a cap on the scores
+// (0: none), sigmoid weights with a bias per query head (head_bias float32 [Hq] or null) instead of the softmax.
+MIE_EXPORT int mie_paged_attention_scored(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                          int dtype, const int* block_tables, int max_blocks, const int* token_row,
+                                          const int* positions, int tokens, int Hq, int Hkv, int D, int page, float scale,
+                                          int window, int has_sink, float sink, int chunk, float softcap, int sigmoid,
+                                          const float* head_bias, hipStream_t stream) {
+  return paged_attention_launch(q, q_stride, k_cache, v_cache, out, dtype, block_tables, max_blocks, token_row, positions,
+                                tokens, Hq, Hkv, D, page, scale, window, has_sink, sink, chunk, softcap, sigmoid, head_bias,
+                                stream);
 }

@@ -1,5 +1,6 @@
 // Between a q/k/v projection's float32 sums and attention, for mixers that want more than a rotation there:
-// an RMS norm over a token's whole query (key) projection, the rotation of the first numbers of every head by
+// an RMS norm over a token's whole query (key) projection (or head by head, with one weight of a head's size for all
+// heads), the rotation of the first numbers of every head by
 // angles computed here in 32-bit (adjacent pairs or the two halves of the turned part), a temperature a query
 // head, values that are the keys as projected, and heads kept in the cache at a padded size.
 //
@@ -14,6 +15,7 @@ enum { LAYOUT_INTERLEAVED = 0, LAYOUT_HALF = 1 };
 struct FinishArgs {
   const float* sums; long ld; int q_col, k_col, v_col;      // v_col < 0: the values are the keys as projected
   const float* q_norm; const float* k_norm; float eps;
+  int norm_per_head;            // the norms are taken head by head; q_norm and k_norm hold dim numbers each
   const float* inv_freq; int nf, layout;
   const float* q_head_scale;
   const int* positions; const int* slots;
@@ -32,12 +34,12 @@ qkv_finish_kernel(FinishArgs a) {
   const float* __restrict__ k = row + a.k_col;
   const int nq = a.Hq * a.dim, nk = a.Hkv * a.dim;
   float rq = 1.f, rk = 1.f;
-  if (a.q_norm) {
+  if (a.q_norm && !a.norm_per_head) {
     float ss = 0.f;
     for (int i = threadIdx.x; i < nq; i += blockDim.x) ss = fmaf(q[i], q[i], ss);
     rq = 1.0f / sqrtf(block_sum(ss, scratch) / (float)nq + a.eps);
   }
-  if (a.k_norm) {
+  if (a.k_norm && !a.norm_per_head) {
     float ss = 0.f;
     for (int i = threadIdx.x; i < nk; i += blockDim.x) ss = fmaf(k[i], k[i], ss);
     rk = 1.0f / sqrtf(block_sum(ss, scratch) / (float)nk + a.eps);
@@ -62,8 +64,13 @@ qkv_finish_kernel(FinishArgs a) {
     const int h = is_q ? job : job - a.Hq;
     const float* __restrict__ x = (is_q ? q : k) + (size_t)h * a.dim;
     const float* __restrict__ w = is_q ? a.q_norm : a.k_norm;
-    if (w) w += (size_t)h * a.dim;
-    const float r = is_q ? rq : rk;
+    if (w && !a.norm_per_head) w += (size_t)h * a.dim;
+    float r = is_q ? rq : rk;
+    if (w && a.norm_per_head) {       // the wave owns the head: its root mean square by a sum over the lanes
+      float ss = 0.f;
+      for (int d = lane; d < a.dim; d += 64) ss = fmaf(x[d], x[d], ss);
+      r = 1.0f / sqrtf(wave_sum(ss) / (float)a.dim + a.eps);
+    }
     const float mult = is_q && a.q_head_scale ? a.q_head_scale[h] : 1.f;
     TO* __restrict__ dst = is_q ? qo + (size_t)h * a.P : kc + ((pg * a.Hkv + h) * a.page + off) * a.P;
     for (int i = lane; i < a.nf; i += 64) {
@@ -89,7 +96,7 @@ qkv_finish_kernel(FinishArgs a) {
 MIE_EXPORT const char* attention_prep_last_error() { return g_mie_error; }
 
 MIE_EXPORT int mie_qkv_finish(const float* sums, long ld, int q_col, int k_col, int v_col, const float* q_norm,
-                              const float* k_norm, float eps, const float* inv_freq, int nf, int layout,
+                              const float* k_norm, float eps, int norm_per_head, const float* inv_freq, int nf, int layout,
                               const float* q_head_scale, const int* positions, const int* slots, void* q_out, void* k_cache,
                               void* v_cache, int dtype, int tokens, int Hq, int Hkv, int dim, int vdim, int P, int page,
                               hipStream_t s) {
@@ -99,7 +106,7 @@ MIE_EXPORT int mie_qkv_finish(const float* sums, long ld, int q_col, int k_col, 
   if (2 * nf > dim || nf < 0 || (nf > 0 && !inv_freq)) MIE_FAIL("qkv_finish: %d turned pairs in heads of %d", nf, dim);
   if (layout != LAYOUT_INTERLEAVED && layout != LAYOUT_HALF) MIE_FAIL("qkv_finish: layout code %d", layout);
   if (v_col < 0 && vdim != dim) MIE_FAIL("qkv_finish: values that are the keys have their size");
-  FinishArgs a{sums, ld, q_col, k_col, v_col, q_norm, k_norm, eps, inv_freq, nf, layout, q_head_scale, positions, slots,
+  FinishArgs a{sums, ld, q_col, k_col, v_col, q_norm, k_norm, eps, norm_per_head, inv_freq, nf, layout, q_head_scale, positions, slots,
                q_out, k_cache, v_cache, Hq, Hkv, dim, vdim, P, page};
   const size_t lds = (size_t)2 * (nf > 0 ? nf : 1) * sizeof(float);
   // few tokens: several workgroups a token, so that a decode step's few rows are spread over the GPU

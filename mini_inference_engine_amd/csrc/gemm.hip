@@ -221,3 +221,65 @@ MIE_EXPORT int mie_act_mul(const void* gu, long ld_in, void* out, long ld_out, i
   MIE_CHECK_LAUNCH("act_mul");
   return 0;
 }
+
+// ---- elementwise steps on a product's float32 sums, rounded once on the way out
+// act_store: out[r, i] = act(in[r, i]).  clamped_glu: in holds gate sums [0, inner) and up sums [inner, 2 inner) of a
+// row; out[r, i] = g * sigmoid(alpha g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit).
+template <typename TO>
+__global__ void __launch_bounds__(256)
+act_store_kernel(const float* __restrict__ in, long ld_in, TO* __restrict__ out, long ld_out, int rows, int n, int act) {
+  const size_t total = (size_t)rows * n;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
+    const size_t r = e / n, i = e - r * n;
+    out[r * ld_out + i] = from_float<TO>(mie_act(in[r * ld_in + i], act));
+  }
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(256)
+clamped_glu_kernel(const float* __restrict__ in, long ld_in, TO* __restrict__ out, long ld_out, int rows, int inner,
+                   float limit, float alpha) {
+  const size_t total = (size_t)rows * inner;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
+    const size_t r = e / inner, i = e - r * inner;
+    const float g = fminf(in[r * ld_in + i], limit);
+    const float u = fminf(fmaxf(in[r * ld_in + inner + i], -limit), limit);
+    out[r * ld_out + i] = from_float<TO>(g * mie_sigmoid(alpha * g) * (u + 1.0f));
+  }
+}
+
+MIE_EXPORT int mie_act_store(const float* in, long ld_in, void* out, long ld_out, int out_dtype, int rows, int n, int act,
+                             hipStream_t s) {
+  if (rows <= 0 || n <= 0) return 0;
+  if (act < MIE_ACT_NONE || act > MIE_ACT_RELU2) MIE_FAIL("act_store: activation code %d", act);
+  if (ld_in < n || ld_out < n) MIE_FAIL("act_store: leading dims %ld, %ld for %d columns", ld_in, ld_out, n);
+  const size_t total = (size_t)rows * n;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 16384) blocks = 16384;
+  if (out_dtype == MIE_F32)
+    hipLaunchKernelGGL(act_store_kernel<float>, dim3(blocks), dim3(256), 0, s, in, ld_in, (float*)out, ld_out, rows, n, act);
+  else if (out_dtype == MIE_BF16)
+    hipLaunchKernelGGL(act_store_kernel<bf16>, dim3(blocks), dim3(256), 0, s, in, ld_in, (bf16*)out, ld_out, rows, n, act);
+  else
+    MIE_FAIL("act_store: dtype code %d", out_dtype);
+  MIE_CHECK_LAUNCH("act_store");
+  return 0;
+}
+
+MIE_EXPORT int mie_clamped_glu(const float* in, long ld_in, void* out, long ld_out, int out_dtype, int rows, int inner,
+                               float limit, float alpha, hipStream_t s) {
+  if (rows <= 0 || inner <= 0) return 0;
+  if (ld_in < 2L * inner || ld_out < inner) MIE_FAIL("clamped_glu: leading dims %ld, %ld for inner size %d", ld_in, ld_out, inner);
+  if (!(limit > 0.f)) MIE_FAIL("clamped_glu: limit %g", (double)limit);
+  const size_t total = (size_t)rows * inner;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 16384) blocks = 16384;
+  if (out_dtype == MIE_F32)
+    hipLaunchKernelGGL(clamped_glu_kernel<float>, dim3(blocks), dim3(256), 0, s, in, ld_in, (float*)out, ld_out, rows, inner, limit, alpha);
+  else if (out_dtype == MIE_BF16)
+    hipLaunchKernelGGL(clamped_glu_kernel<bf16>, dim3(blocks), dim3(256), 0, s, in, ld_in, (bf16*)out, ld_out, rows, inner, limit, alpha);
+  else
+    MIE_FAIL("clamped_glu: dtype code %d", out_dtype);
+  MIE_CHECK_LAUNCH("clamped_glu");
+  return 0;
+}

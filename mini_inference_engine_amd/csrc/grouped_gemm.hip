@@ -380,46 +380,74 @@ MIE_EXPORT int mie_grouped_linear(const void* A, int a_dtype, long lda, long a_g
   MIE_FAIL("grouped_linear: dtype codes A %d, W %d", a_dtype, w_dtype);
 }
 
-// ---- router: the `top` largest of logits[t, :] + bias (lowest index first among equals), in falling order, and
-// the softmax over those alone.  One thread a token.
+// ---- router, one thread a token.  over_all == 0: the `top` largest of logits[t, :] + bias (lowest index first among
+// equals), in falling order, and the softmax over those alone.  over_all != 0: scores = softmax of logits + bias over
+// all E; chosen are the `top` largest of scores + choice_bias (same order rules); the shares are the chosen ones'
+// scores as they are.
 #define ROUTE_MAX_TOP 16
 __global__ void route_topk_kernel(const float* __restrict__ logits, long ld, const float* __restrict__ bias,
-                                  int* __restrict__ experts, float* __restrict__ shares, int T, int E, int top) {
+                                  const float* __restrict__ choice_bias, int over_all, int* __restrict__ experts,
+                                  float* __restrict__ shares, int T, int E, int top) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const float* z = logits + (size_t)t * ld;
+  float largest = 0.f, total = 1.f;
+  if (over_all) {
+    largest = -INFINITY;
+    for (int e = 0; e < E; ++e) largest = fmaxf(largest, z[e] + (bias ? bias[e] : 0.f));
+    total = 0.f;
+    for (int e = 0; e < E; ++e) total += expf(z[e] + (bias ? bias[e] : 0.f) - largest);
+  }
   int chosen[ROUTE_MAX_TOP];
   float val[ROUTE_MAX_TOP];
   for (int j = 0; j < top; ++j) {
     int best = -1;
-    float bv = 0.f;
+    float bv = 0.f, bs = 0.f;
     for (int e = 0; e < E; ++e) {
       bool taken = false;
       for (int i = 0; i < j; ++i) taken |= chosen[i] == e;
       if (taken) continue;
-      const float v = z[e] + (bias ? bias[e] : 0.f);
-      if (best < 0 || v > bv) { best = e; bv = v; }
+      float v = z[e] + (bias ? bias[e] : 0.f), sc = v;
+      if (over_all) {
+        sc = expf(v - largest) / total;
+        v = sc + (choice_bias ? choice_bias[e] : 0.f);
+      }
+      if (best < 0 || v > bv) { best = e; bv = v; bs = sc; }
     }
     chosen[j] = best;
-    val[j] = bv;
+    val[j] = bs;
   }
-  float sum = 0.f;
-  const float largest = val[0];
-  for (int j = 0; j < top; ++j) { val[j] = expf(val[j] - largest); sum += val[j]; }
+  if (!over_all) {
+    float sum = 0.f;
+    const float first = val[0];
+    for (int j = 0; j < top; ++j) { val[j] = expf(val[j] - first); sum += val[j]; }
+    for (int j = 0; j < top; ++j) val[j] /= sum;
+  }
   for (int j = 0; j < top; ++j) {
     experts[(size_t)t * top + j] = chosen[j];
-    shares[(size_t)t * top + j] = val[j] / sum;
+    shares[(size_t)t * top + j] = val[j];
   }
+}
+
+static int route_topk_launch(const float* logits, long ld, const float* bias, const float* choice_bias, int over_all,
+                             int* experts, float* shares, int T, int E, int top, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (E <= 0 || top <= 0 || top > E || top > ROUTE_MAX_TOP) MIE_FAIL("route_topk: top %d of %d experts (at most %d)", top, E, ROUTE_MAX_TOP);
+  if (ld < E) MIE_FAIL("route_topk: row stride %ld < %d", ld, E);
+  hipLaunchKernelGGL(route_topk_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, ld, bias, choice_bias, over_all, experts,
+                     shares, T, E, top);
+  MIE_CHECK_LAUNCH("route_topk");
+  return 0;
 }
 
 MIE_EXPORT int mie_route_topk(const float* logits, long ld, const float* bias, int* experts, float* shares, int T, int E,
                               int top, hipStream_t s) {
-  if (T <= 0) return 0;
-  if (E <= 0 || top <= 0 || top > E || top > ROUTE_MAX_TOP) MIE_FAIL("route_topk: top %d of %d experts (at most %d)", top, E, ROUTE_MAX_TOP);
-  if (ld < E) MIE_FAIL("route_topk: row stride %ld < %d", ld, E);
-  hipLaunchKernelGGL(route_topk_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, ld, bias, experts, shares, T, E, top);
-  MIE_CHECK_LAUNCH("route_topk");
-  return 0;
+  return route_topk_launch(logits, ld, bias, nullptr, 0, experts, shares, T, E, top, s);
+}
+
+MIE_EXPORT int mie_route_topk_all(const float* logits, long ld, const float* bias, const float* choice_bias, int* experts,
+                                  float* shares, int T, int E, int top, hipStream_t s) {
+  return route_topk_launch(logits, ld, bias, choice_bias, 1, experts, shares, T, E, top, s);
 }
 
 // ---- sort the n = T * top (token, choice) pairs by expert: offs [E + 1] (where each expert's pairs start in the
@@ -464,14 +492,22 @@ MIE_EXPORT int mie_moe_align(const int* experts, int n, int E, int* offs, int* s
   return 0;
 }
 
-// ---- out[t, :] = sum over a token's choices j, in order, of shares[t, j] * y[place[t * top + j], :]
+// ---- out[t, :] = sum over a token's choices j, in order, of shares[t, j] * y[place[t * top + j], :].  With x given,
+// a choice of an expert >= identity_from stands for the token's own input: its term is shares[t, j] * x[t, :] and its
+// row of y is not read.
+template <typename TX>
 __global__ void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, const float* __restrict__ shares,
-                                   float* __restrict__ out, int width, int top) {
+                                   float* __restrict__ out, int width, int top, const int* __restrict__ experts,
+                                   int identity_from, const TX* __restrict__ x, long ldx) {
   const int t = blockIdx.x;
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
     float acc = 0.f;
-    for (int j = 0; j < top; ++j)
-      acc = fmaf(shares[(size_t)t * top + j], y[(size_t)place[(size_t)t * top + j] * width + c], acc);
+    for (int j = 0; j < top; ++j) {
+      const size_t at = (size_t)t * top + j;
+      const bool same = x != nullptr && experts[at] >= identity_from;
+      const float v = same ? to_float(x[(size_t)t * ldx + c]) : y[(size_t)place[at] * width + c];
+      acc = fmaf(shares[at], v, acc);
+    }
     out[(size_t)t * width + c] = acc;
   }
 }
@@ -481,7 +517,29 @@ MIE_EXPORT int mie_moe_combine(const float* y, const int* place, const float* sh
   if (T <= 0 || width <= 0) return 0;
   if (top <= 0) MIE_FAIL("moe_combine: top %d", top);
   int by = (width + 255) / 256;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, by > 16 ? 16 : by), dim3(256), 0, s, y, place, shares, out, width, top);
+  hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(T, by > 16 ? 16 : by), dim3(256), 0, s, y, place, shares, out, width, top,
+                     (const int*)nullptr, 0, (const float*)nullptr, 0L);
+  MIE_CHECK_LAUNCH("moe_combine");
+  return 0;
+}
+
+MIE_EXPORT int mie_moe_combine_identity(const float* y, const int* place, const float* shares, float* out, int T, int width,
+                                        int top, const int* experts, int identity_from, const void* x, int x_dtype, long ldx,
+                                        hipStream_t s) {
+  if (T <= 0 || width <= 0) return 0;
+  if (top <= 0 || !experts || !x || ldx < width || identity_from < 0)
+    MIE_FAIL("moe_combine: top %d, identity experts from %d, input rows %ld apart", top, identity_from, ldx);
+  if (identity_from > 0 && !y) MIE_FAIL("moe_combine: experts without outputs");
+  int by = (width + 255) / 256;
+  dim3 grid(T, by > 16 ? 16 : by);
+  if (x_dtype == MIE_F32)
+    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, dim3(256), 0, s, y, place, shares, out, width, top, experts,
+                       identity_from, (const float*)x, ldx);
+  else if (x_dtype == MIE_BF16)
+    hipLaunchKernelGGL(moe_combine_kernel<bf16>, grid, dim3(256), 0, s, y, place, shares, out, width, top, experts,
+                       identity_from, (const bf16*)x, ldx);
+  else
+    MIE_FAIL("moe_combine: dtype code %d", x_dtype);
   MIE_CHECK_LAUNCH("moe_combine");
   return 0;
 }

@@ -409,6 +409,16 @@ class HipBackend(KernelBackend):
                                            intermediate, self.ACT_CODES[activation], self._stream()))
         return out
 
+    def linear_act(self, x, w, activation="relu2"):
+        if activation not in self.ACT_CODES:
+            raise ValueError(f"linear_act: activation {activation!r}")
+        sums = self.linear(x, w, out_dtype=torch.float32)
+        out = torch.empty(sums.shape, dtype=self.act_dtype, device=sums.device)
+        lib = self.lib("gemm")
+        library.check(lib, lib.mie_act_store(_ptr(sums), sums.stride(0), _ptr(out), out.stride(0), _code(out.dtype),
+                                             sums.shape[0], sums.shape[1], self.ACT_CODES[activation], self._stream()))
+        return out
+
     def scale_(self, t, factor):
         self._on_device(t)
         if t.dtype != torch.float32 or not t.is_contiguous():
@@ -417,7 +427,7 @@ class HipBackend(KernelBackend):
         library.check(lib, lib.mie_scale(_ptr(t), t.numel(), float(factor), self._stream()))
         return t
 
-    def branch_norm_add(self, y, stream, weight, eps):
+    def branch_norm_add(self, y, stream, weight, eps, copy=True):
         self._on_device(y, stream, weight)
         if stream.dtype != torch.float32 or stream.dim() != 2 or not stream.is_contiguous():
             raise ValueError("branch_norm_add: the stream must be contiguous float32 [T, width]")
@@ -427,13 +437,17 @@ class HipBackend(KernelBackend):
                 raise ValueError(f"branch_norm_add: y {tuple(y.shape)} does not match the stream {(T, W)}")
             if weight is None or tuple(weight.shape) != (W,) or not weight.is_contiguous():
                 raise ValueError(f"branch_norm_add: a contiguous weight of {W}")
-        copy = None if self.act_dtype == torch.float32 else torch.empty((T, W), dtype=self.act_dtype, device=stream.device)
+        want_copy = copy
+        copy = None if self.act_dtype == torch.float32 or not want_copy else torch.empty((T, W), dtype=self.act_dtype,
+                                                                                         device=stream.device)
         if y is not None or copy is not None:
             lib = self.lib("embed_norm")
             library.check(lib, lib.mie_branch_norm_add(
                 _ptr(y), _code(y.dtype) if y is not None else F32, _ptr(stream), _ptr(weight),
                 _code(weight.dtype) if weight is not None else F32, _ptr(copy), _code(copy.dtype) if copy is not None else F32,
                 T, W, float(eps), self._stream()))
+        if not want_copy:
+            return None
         return stream if copy is None else copy
 
     @staticmethod
@@ -631,8 +645,10 @@ class HipBackend(KernelBackend):
         return out
 
     # ---- routed experts
-    def route_topk(self, logits, bias, top):
-        self._on_device(logits, bias)
+    def route_topk(self, logits, bias, top, over="chosen", choice_bias=None):
+        self._on_device(logits, bias, choice_bias)
+        if over not in ("chosen", "all") or (choice_bias is not None and over != "all"):
+            raise ValueError(f"route_topk: shares over {over!r} (chosen or all; a choice bias goes with all)")
         if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
             raise ValueError("route_topk: logits must be float32 [T, experts] with unit inner stride")
         T, E = logits.shape
@@ -643,39 +659,72 @@ class HipBackend(KernelBackend):
         experts = torch.empty((T, top), dtype=torch.int32, device=logits.device)
         shares = torch.empty((T, top), dtype=torch.float32, device=logits.device)
         lib = self.lib("grouped_gemm")
+        if over == "all":
+            if choice_bias is not None:
+                self._f32_vector(choice_bias, E, "route_topk: choice bias")
+            library.check(lib, lib.mie_route_topk_all(_ptr(logits), logits.stride(0), _ptr(bias), _ptr(choice_bias), _ptr(experts),
+                                                      _ptr(shares), T, E, top, self._stream()))
+            return experts, shares
         library.check(lib, lib.mie_route_topk(_ptr(logits), logits.stride(0), _ptr(bias), _ptr(experts), _ptr(shares), T, E, top,
                                               self._stream()))
         return experts, shares
 
-    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2"):
+    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None):
         self._on_device(x, experts, shares, w_up, w_down)
         _rows_ok(x, "routed_experts: x")
         T, W = x.shape
-        if w_up.dim() != 3 or w_down.dim() != 3 or not (w_up.is_contiguous() and w_down.is_contiguous()):
-            raise ValueError("routed_experts: contiguous [experts, ff, width] and [experts, width, ff]")
-        E, ff, _ = w_up.shape
-        if w_up.shape[2] != W or tuple(w_down.shape) != (E, W, ff):
-            raise ValueError(f"routed_experts: w_up {tuple(w_up.shape)}, w_down {tuple(w_down.shape)} for width {W}")
         top = experts.shape[1]
         if experts.dtype != torch.int32 or tuple(experts.shape) != (T, top) or not experts.is_contiguous() \
                 or shares.dtype != torch.float32 or tuple(shares.shape) != (T, top) or not shares.is_contiguous():
             raise ValueError("routed_experts: experts int32 [T, top] and shares float32 [T, top], contiguous")
-        if activation not in self.ACT_CODES:
-            raise ValueError(f"routed_experts: activation {activation!r}")
-        n = T * top
         dev = x.device
-        offs = torch.empty(E + 1, dtype=torch.int32, device=dev)
+        lib = self.lib("grouped_gemm")
+        out = torch.empty((T, W), dtype=torch.float32, device=dev)
+        n = T * top
+        if w_up is None:            # every choice stands for the token's own input
+            if identity_from != 0 or w_down is not None:
+                raise ValueError("routed_experts: experts without matrices must all be identity experts (identity_from 0)")
+            library.check(lib, lib.mie_moe_combine_identity(None, _ptr(experts), _ptr(shares), _ptr(out), T, W, top, _ptr(experts),
+                                                            0, _ptr(x), _code(x.dtype), x.stride(0), self._stream()))
+            return out
+        if w_up.dim() != 3 or w_down.dim() != 3 or not (w_up.is_contiguous() and w_down.is_contiguous()):
+            raise ValueError("routed_experts: contiguous [experts, ff, width] and [experts, width, ff]")
+        E, up_rows, _ = w_up.shape
+        ff = up_rows if gated is None else up_rows // 2
+        if w_up.shape[2] != W or tuple(w_down.shape) != (E, W, ff) or (gated is not None and up_rows != 2 * ff):
+            raise ValueError(f"routed_experts: w_up {tuple(w_up.shape)}, w_down {tuple(w_down.shape)} for width {W}")
+        if identity_from is not None and identity_from != E:
+            raise ValueError(f"routed_experts: identity experts from {identity_from} on, but {E} experts have matrices")
+        if gated is None and activation not in self.ACT_CODES:
+            raise ValueError(f"routed_experts: activation {activation!r}")
+        groups = E if identity_from is None else E + 1      # one more group behind the experts holds every identity choice
+        offs = torch.empty(groups + 1, dtype=torch.int32, device=dev)
         order = torch.empty(n, dtype=torch.int32, device=dev)
         place = torch.empty(n, dtype=torch.int32, device=dev)
-        lib = self.lib("grouped_gemm")
-        library.check(lib, lib.mie_moe_align(_ptr(experts), n, E, _ptr(offs), _ptr(order), _ptr(place), self._stream()))
+        # identity choices are sorted behind the experts' (the sort clamps every choice >= the last group into it), so
+        # the grouped products, which walk the first E groups, never see them
+        library.check(lib, lib.mie_moe_align(_ptr(experts), n, groups, _ptr(offs), _ptr(order), _ptr(place), self._stream()))
         hidden = torch.empty((n, ff), dtype=self.act_dtype, device=dev)
-        self._grouped(x, x.stride(0), 0, 1, w_up, W, ff * W, hidden, ff, 0, n, ff, W, E, offs=offs, gather=order, gather_div=top,
-                      act=activation)
+        if gated is None:
+            self._grouped(x, x.stride(0), 0, 1, w_up, W, ff * W, hidden, ff, 0, n, ff, W, E, offs=offs, gather=order,
+                          gather_div=top, act=activation)
+        else:
+            limit, alpha = gated
+            gu = torch.empty((n, 2 * ff), dtype=torch.float32, device=dev)
+            self._grouped(x, x.stride(0), 0, 1, w_up, W, 2 * ff * W, gu, 2 * ff, 0, n, 2 * ff, W, E, offs=offs, gather=order,
+                          gather_div=top)
+            glib = self.lib("gemm")
+            # rows of identity choices hold whatever was there: the function of it is never read
+            library.check(glib, glib.mie_clamped_glu(_ptr(gu), gu.stride(0), _ptr(hidden), hidden.stride(0), _code(hidden.dtype),
+                                                     n, ff, float(limit), float(alpha), self._stream()))
         y = torch.empty((n, W), dtype=torch.float32, device=dev)
         self._grouped(hidden, ff, 0, 1, w_down, ff, W * ff, y, W, 0, n, W, ff, E, offs=offs)
-        out = torch.empty((T, W), dtype=torch.float32, device=dev)
-        library.check(lib, lib.mie_moe_combine(_ptr(y), _ptr(place), _ptr(shares), _ptr(out), T, W, top, self._stream()))
+        if identity_from is None:
+            library.check(lib, lib.mie_moe_combine(_ptr(y), _ptr(place), _ptr(shares), _ptr(out), T, W, top, self._stream()))
+        else:
+            library.check(lib, lib.mie_moe_combine_identity(_ptr(y), _ptr(place), _ptr(shares), _ptr(out), T, W, top,
+                                                            _ptr(experts), E, _ptr(x), _code(x.dtype), x.stride(0),
+                                                            self._stream()))
         return out
 
     # ---- a short convolution on a mixer's input, attention from one product's sums, the delta rule
@@ -738,7 +787,8 @@ class HipBackend(KernelBackend):
     DELTA_CHUNKED_MAX_DIM = 128   # wider heads always run whole (the fold keeps a chunk's d x d matrix in the LDS)
 
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
-                   layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None):
+                   layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None,
+                   norm_per_head=False):
         self._on_device(sums, positions, inv_freq, k_cache, v_cache, slot_mapping, q_norm, k_norm, q_head_scale)
         Hq, Hkv, P, T = num_q_heads, num_kv_heads, padded_dim, sums.shape[0]
         if layout not in self.LAYOUTS:
@@ -759,7 +809,8 @@ class HipBackend(KernelBackend):
             self._f32_vector(inv_freq, nf, "qkv_finish: inv_freq")
         if 2 * nf > dim:
             raise ValueError(f"qkv_finish: {nf} turned pairs in heads of {dim}")
-        for name, t, n in (("q_norm", q_norm, Hq * dim), ("k_norm", k_norm, Hkv * dim), ("q_head_scale", q_head_scale, Hq)):
+        for name, t, n in (("q_norm", q_norm, dim if norm_per_head else Hq * dim),
+                           ("k_norm", k_norm, dim if norm_per_head else Hkv * dim), ("q_head_scale", q_head_scale, Hq)):
             if t is not None:
                 self._f32_vector(t, n, f"qkv_finish: {name}")
         for name, t in (("positions", positions), ("slot_mapping", slot_mapping)):
@@ -770,7 +821,7 @@ class HipBackend(KernelBackend):
         lib = self.lib("attention_prep")
         library.check(lib, lib.mie_qkv_finish(
             _ptr(sums), sums.stride(0), q_col, k_col, -1 if v_col is None else v_col, _ptr(q_norm), _ptr(k_norm), float(eps),
-            _ptr(inv_freq), nf, self.LAYOUTS[layout], _ptr(q_head_scale), _ptr(positions), _ptr(slot_mapping), _ptr(q),
+            int(bool(norm_per_head)), _ptr(inv_freq), nf, self.LAYOUTS[layout], _ptr(q_head_scale), _ptr(positions), _ptr(slot_mapping), _ptr(q),
             _ptr(k_cache), _ptr(v_cache), _code(self.act_dtype), T, Hq, Hkv, dim, vdim, P, page, self._stream()))
         return q
 
@@ -1029,9 +1080,25 @@ class HipBackend(KernelBackend):
         return out
 
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
-                        window, sink=None, force_generic: bool = False, num_splits: int | None = None):
+                        window, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None,
+                        force_generic: bool = False, num_splits: int | None = None):
         Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
         has_sink, sink = int(sink is not None), float(sink or 0.0)
+        if weights not in ("softmax", "sigmoid"):
+            raise ValueError(f"paged_attention: weights {weights!r} (softmax or sigmoid)")
+        sigmoid = weights == "sigmoid"
+        if sigmoid and has_sink:
+            raise ValueError("paged_attention: a sink belongs to a softmax")
+        if (chunk is not None and chunk < 1) or (softcap is not None and not softcap > 0):
+            raise ValueError(f"paged_attention: chunk {chunk}, score cap {softcap}")
+        if head_bias is not None:
+            if not sigmoid:
+                raise ValueError("paged_attention: a bias per head goes with sigmoid weights")
+            self._on_device(head_bias)
+            self._f32_vector(head_bias, Hq, "paged_attention: head_bias")
+        scored = sigmoid or softcap is not None or chunk is not None
+        if scored and not sigmoid:
+            force_generic = True            # a capped or chunked softmax: the 32-bit kernel computes it
         if isinstance(qkv, ProjectionSums):
             out = self._decode_attention_from_sums(qkv, Hq, Hkv, D, k_cache, v_cache, group, step, scale, window,
                                                    force_generic or num_splits is not None or bool(has_sink))
@@ -1044,6 +1111,8 @@ class HipBackend(KernelBackend):
         done = 0
         if D > 256:
             force_generic = True            # beyond the matrix-core kernels' head sizes: the 32-bit kernel takes up to 1,024
+        if sigmoid:
+            force_generic = True
         if qkv.dtype == torch.bfloat16 and not force_generic and step.num_decode_rows > 0:
             done = step.num_decode_rows        # single-token rows lead the batch: token t is row t
             lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))
@@ -1083,11 +1152,15 @@ class HipBackend(KernelBackend):
         if done < T:
             lib = self.lib("attention")
             esz = qkv.element_size()
-            library.check(lib, lib.mie_paged_attention(
-                c_void_p(qkv.data_ptr() + done * qkv.stride(0) * esz), qkv.stride(0), _ptr(k_cache), _ptr(v_cache),
-                c_void_p(out.data_ptr() + done * Hq * D * esz), _code(qkv.dtype), _ptr(bt), bt.shape[1],
-                c_void_p(step.token_row.data_ptr() + done * 4), c_void_p(step.positions.data_ptr() + done * 4),
-                T - done, Hq, Hkv, D, page, float(scale), int(window or 0), has_sink, sink, self._stream()))
+            args = (c_void_p(qkv.data_ptr() + done * qkv.stride(0) * esz), qkv.stride(0), _ptr(k_cache), _ptr(v_cache),
+                    c_void_p(out.data_ptr() + done * Hq * D * esz), _code(qkv.dtype), _ptr(bt), bt.shape[1],
+                    c_void_p(step.token_row.data_ptr() + done * 4), c_void_p(step.positions.data_ptr() + done * 4),
+                    T - done, Hq, Hkv, D, page, float(scale), int(window or 0), has_sink, sink)
+            if scored:
+                library.check(lib, lib.mie_paged_attention_scored(*args, int(chunk or 0), float(softcap or 0.0), int(sigmoid),
+                                                                  _ptr(head_bias), self._stream()))
+            else:
+                library.check(lib, lib.mie_paged_attention(*args, self._stream()))
         return out
 
     def sample(self, logits, temperatures, seeds, counters, out=None):

@@ -26,12 +26,16 @@ register_kernel_module("gemm", {
     "mie_gemm_nt": [P, I, L, P, I, L, P, I, L, P, I, I, I, P],
     "mie_silu_mul": [P, L, P, L, I, I, I, P],
     "mie_act_mul": [P, L, P, L, I, I, I, I, P],
+    "mie_act_store": [P, L, P, L, I, I, I, I, P],
+    "mie_clamped_glu": [P, L, P, L, I, I, I, F, F, P],
 })
 register_kernel_module("grouped_gemm", {
     "mie_grouped_linear": [P, I, L, L, I, P, I, L, L, P, I, L, L, P, P, L, P, P, I, I, I, I, I, I, P, P],
     "mie_route_topk": [P, L, P, P, P, I, I, I, P],
+    "mie_route_topk_all": [P, L, P, P, P, P, I, I, I, P],
     "mie_moe_align": [P, I, I, P, P, P, P],
     "mie_moe_combine": [P, P, P, P, I, I, I, P],
+    "mie_moe_combine_identity": [P, P, P, P, I, I, I, P, I, P, I, L, P],
 })
 register_kernel_module("latent_attention", {
     "mie_latent_kv_store": [P, L, P, I, F, P, P, I, P, P, I, P, I, I, I, I, I, P, P, P, I, P],
@@ -44,7 +48,7 @@ register_kernel_module("recurrence", {
     "mie_residual_conv": [P, P, P, P, P, P, P, I, I, I, I, I, P],
 })
 register_kernel_module("attention_prep", {
-    "mie_qkv_finish": [P, L, I, I, I, P, P, F, P, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+    "mie_qkv_finish": [P, L, I, I, I, P, P, F, I, P, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
     "mie_head_gate": [P, I, P, L, I, I, I, P],
 })
 register_kernel_module("delta_rule", {
@@ -52,6 +56,7 @@ register_kernel_module("delta_rule", {
 })
 register_kernel_module("attention", {
     "mie_paged_attention": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, I, F, P],
+    "mie_paged_attention_scored": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, I, F, I, F, I, P, P],
 })
 register_kernel_module("sampling", {
     "mie_sample": [P, L, P, P, P, P, I, I, P],
