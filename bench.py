@@ -3,7 +3,7 @@ Llama-2-7B or Llama-3-8B), random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--shape tinyllama] [--context N] [--layers L]
     python bench.py --kernels [--shape ...] [--batch 8] [--context N]     each dominant kernel alone
-    python bench.py --design zifelorn|vezodra [--design-sizes 1024,2048] [--layers R] [--batch 8] [--context 1024]
+    python bench.py --design zifelorn|vezodra|mutusun [--design-sizes 1024,2048] [--layers R] [--batch 8] [--context 1024]
                                                  that design beside Llama at equal layer sizes (R runs of its layers)
 
 A step is one decode step of the engine (schedule, batch, captured forward, sampling,
@@ -449,10 +449,25 @@ VEZODRA_SIZES = {
 }
 
 
+# Mutusun layer sizes of the same widths: a run of three layers is chunked sigmoid attention + dense, the same attention
+# + gated experts (four of them a token, together as large as the dense feed-forward, among the experts and two
+# identity outputs), and that routed layer once more with the same tensors and a cache of its own.
+MUTUSUN_SIZES = {
+    "1024": dict(vocab=32000, width=1024, heads=16, kv_heads=4, dim=64, chunk=1024, ff=2816, experts=8, identity=2, top=4,
+                 expert_ff=704),
+    "2048": dict(vocab=32000, width=2048, heads=32, kv_heads=8, dim=64, chunk=1024, ff=5632, experts=16, identity=2, top=4,
+                 expert_ff=1408),
+}
+
+
 def design_configs(design: str, size: str, repeats: int):
     """(the design's configuration, Llama's of the same width, head count, feed-forward size, vocabulary and layer count)."""
-    from mini_inference_engine_amd.config import LlamaConfig, VezodraConfig, ZifelornConfig
-    if design == "vezodra":
+    from mini_inference_engine_amd.config import LlamaConfig, MutusunConfig, VezodraConfig, ZifelornConfig
+    if design == "mutusun":
+        from mini_inference_engine_amd.models.mutusun import _shape
+        z = MUTUSUN_SIZES[size]
+        cfg, layers = MutusunConfig.from_dict(_shape(repeats=repeats, shared=1, **z)), 3 * repeats
+    elif design == "vezodra":
         from mini_inference_engine_amd.models.vezodra import _shape
         z = VEZODRA_SIZES[size]
         cfg, layers = VezodraConfig.from_dict(_shape(repeats=repeats, times=1, **z)), 3 * repeats
@@ -503,7 +518,7 @@ def measure_designs(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["zifelorn", "vezodra"], default=None,
+    ap.add_argument("--design", choices=["zifelorn", "vezodra", "mutusun"], default=None,
                     help="instead of the default workload: that design beside Llama at equal layer sizes (decode and prefill)")
     ap.add_argument("--design-sizes", default=None, help="comma-separated widths of --design (default: all of 1024, 2048)")
     ap.add_argument("--gpus", type=int, default=1)

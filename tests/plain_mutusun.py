@@ -79,17 +79,22 @@ def expert(h, W, p, limit):
     return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ W[f"{p}.down"].T
 
 
-def route(h, W, p, top):
+def route(h, W, p, top, margins=None):
     """-> (chosen [n, top], their weights [n, top]): softmax over all router outputs; the choice goes by the
-    scores plus a correction, the weights are the scores themselves, not renormalised."""
+    scores plus a correction, the weights are the scores themselves, not renormalised.  ``margins`` (a list)
+    receives, per token, the gap between the last chosen and the first refused choice score."""
     s = torch.softmax(h @ W[f"{p}.router"].T, dim=-1)
-    chosen = torch.topk(s + W[f"{p}.correction"], top, dim=-1).indices
+    by = s + W[f"{p}.correction"]
+    chosen = torch.topk(by, top, dim=-1).indices
+    if margins is not None and top < by.shape[-1]:
+        ranked = torch.sort(by, dim=-1, descending=True).values
+        margins += (ranked[:, top - 1] - ranked[:, top]).tolist()
     return chosen, torch.gather(s, 1, chosen)
 
 
-def moe_ff(h, W, p, f):
+def moe_ff(h, W, p, f, margins=None):
     E, top = f["router"]["experts"], f["router"]["top"]
-    chosen, weight = route(h, W, p, top)
+    chosen, weight = route(h, W, p, top, margins)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, w in zip(chosen[t].tolist(), weight[t]):
@@ -99,13 +104,13 @@ def moe_ff(h, W, p, f):
     return out
 
 
-def forward(config, weights, ids, streams=None, dtype=torch.float64):
+def forward(config, weights, ids, streams=None, dtype=torch.float64, margins=None):
     W = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = config["norm"]["eps"]
     taps = (config.get("canon") or {}).get("taps")
     s = W["embed"][torch.as_tensor(ids, dtype=torch.long)]
     for i, layer in enumerate(config["layers"]):
-        p = f"l{layer.get('weights_of', i)}"
+        p = f"l{i if layer.get('weights_of') is None else layer['weights_of']}"
         h = rms_norm(s, W[f"{p}.norm1"], eps, one_plus=True)
         if taps:
             h = input_conv(h, W[f"{p}.canon1"])
@@ -117,7 +122,7 @@ def forward(config, weights, ids, streams=None, dtype=torch.float64):
             h = rms_norm(s, W[f"{p}.norm2"], eps, one_plus=True)
             if taps:
                 h = input_conv(h, W[f"{p}.canon2"])
-            y = dense_ff(h, W, f"{p}.mlp") if f["kind"] == "dense" else moe_ff(h, W, f"{p}.mlp", f)
+            y = dense_ff(h, W, f"{p}.mlp") if f["kind"] == "dense" else moe_ff(h, W, f"{p}.mlp", f, margins)
             s = s + rms_norm(y, W[f"{p}.norm2b"], eps, one_plus=True)
         if streams is not None:
             streams.append(s.clone())
