@@ -39,14 +39,18 @@ struct ProjectionSums {
   const int* slots;          // [rows] cache slot of each row's token
 };
 
-template <int NW, bool FROM_SUMS>
+// SIG: sigmoid weights instead of a softmax.  A visible key counts with sigmoid(cap(score) + the head's bias),
+// cap(x) = c tanh(x / c) or x itself; a chunk size n (0: none) hides the keys before floor(position / n) n.  There
+// is no maximum and no denominator: waves and splits simply add up (the merge sees maxima of 0 and one unit sum
+// a workgroup, and the kernel that joins the splits is told not to divide).  scale_log2 then carries the plain scale.
+template <int NW, bool FROM_SUMS, bool SIG = false>
 __global__ void __launch_bounds__(NW * 64)
 decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache, bf16* v_cache,
                         bf16* __restrict__ out, float* __restrict__ o_part,
                         float* __restrict__ lse_part, const int* __restrict__ block_tables, int max_blocks,
                         const int* __restrict__ positions, int Hq, int Hkv, int head_tiles, int page,
                         float scale_log2, int window, int partition, int num_splits, ProjectionSums proj,
-                        float sink_log2) {
+                        float sink_log2, int chunk, float softcap, const float* __restrict__ head_bias) {
   __shared__ float s_m[NW][16], s_l[NW][16], s_M[16], s_L[16];
   __shared__ float s_o[NW][16][D + 1];
   __shared__ __align__(16) bf16 s_q[FROM_SUMS ? 16 : 1][D];
@@ -107,7 +111,7 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
   KeyBlock b0, b1;
   const int pos_raw = positions[b];
   int begin0 = s * partition;               // the split's first key when there is no window
-  if (AHEAD && window <= 0) load_block(b0, begin0 + BLOCK_KEYS * wave);
+  if (AHEAD && window <= 0 && (!SIG || chunk <= 0)) load_block(b0, begin0 + BLOCK_KEYS * wave);
 
   const int pos = pos_raw;
   if (FROM_SUMS) {
@@ -152,7 +156,21 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
       if (head_ok && d0 < D) qf[ks].q = *reinterpret_cast<const uint4*>(&s_q[g][d0]);
     }
   }
-  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  float sg_c1 = 0.f, sg_c2 = 0.f, sg_c3 = 0.f;
+  if constexpr (SIG) {
+    if (chunk > 0 && pos / chunk * chunk > lo) lo = pos / chunk * chunk;
+    const float hb = head_bias ? head_bias[head] : 0.f;
+    const float L2E = 1.4426950408889634f;
+    if (softcap > 0.f) {
+      sg_c1 = 2.f * L2E * scale_log2 / softcap;
+      sg_c2 = 2.f * L2E * softcap;
+      sg_c3 = -L2E * (softcap + hb);
+    } else {
+      sg_c1 = -L2E * scale_log2;
+      sg_c3 = -L2E * hb;
+    }
+  }
   const int begin = (lo & ~(BLOCK_KEYS - 1)) + s * partition;
   const int end = begin + partition < pos + 1 ? begin + partition : pos + 1;
 
@@ -207,6 +225,42 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
         S[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(B.a[t][ks].v, qf[ks].v, S[t], 0, 0, 0);
     }
     const bool partial = blk + BLOCK_KEYS > pos + 1 || blk < lo;
+    if constexpr (SIG) {
+      bool ok[8];
+      float p[8];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = blk + 16 * t + 4 * kb + i;
+          ok[t * 4 + i] = key >= lo && key <= pos;
+          float w;
+          if (softcap > 0.f) {
+            const float r = __builtin_amdgcn_rcpf(1.f + fast_exp2(S[t][i] * sg_c1));
+            w = __builtin_amdgcn_rcpf(1.f + fast_exp2(fmaf(r, sg_c2, sg_c3)));
+          } else {
+            w = __builtin_amdgcn_rcpf(1.f + fast_exp2(fmaf(S[t][i], sg_c1, sg_c3)));
+          }
+          p[t * 4 + i] = ok[t * 4 + i] ? w : 0.f;
+        }
+      Frag pb;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pb.w[j] = pack_bf16(p[2 * j], p[2 * j + 1]);
+      if (partial) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            uint32_t w = B.va[dt].w[j];
+            if (!ok[2 * j]) w &= 0xFFFF0000u;
+            if (!ok[2 * j + 1]) w &= 0x0000FFFFu;
+            B.va[dt].w[j] = w;
+          }
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(B.va[dt].v, pb.v, O[dt], 0, 0, 0);
+      return;
+    }
     // ---- online softmax, one head per lane column
     float sv[8];
     bool ok[8];
@@ -259,7 +313,7 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
   constexpr int STEP = BLOCK_KEYS * NW;     // keys from one block of a wave to its next
   const int first = begin + BLOCK_KEYS * wave;
   if (AHEAD) {
-    if (window > 0) load_block(b0, first);  // with a window the split's start had to wait for the row's length
+    if (window > 0 || (SIG && chunk > 0)) load_block(b0, first);  // with a window the split's start had to wait for the row's length
     const int part_end = begin + partition;   // nothing is asked for beyond the split's own keys
     for (int blk = first; blk < end; blk += 2 * STEP) {
       if (blk + STEP < part_end) load_block(b1, blk + STEP);           // in flight while block 0 is computed
@@ -275,6 +329,10 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
   }
 
   // ---- merge the waves of the workgroup
+  if constexpr (SIG) {
+    m = 0.f;
+    l = wave == 0 ? 1.f : 0.f;
+  }
   if (kb == 0) {
     s_m[wave][col] = m;
     s_l[wave][col] = l;
@@ -325,7 +383,7 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
 // cross the per-XCD L2s, and the device-scope fences that takes cost far more than this launch.)
 __global__ void __launch_bounds__(64)
 merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ lse_part, bf16* __restrict__ out,
-                    int num_splits, float sink_log2) {
+                    int num_splits, float sink_log2, int plain_sum) {
   constexpr int DL = (D + 63) / 64;
   const size_t hh = blockIdx.x;
   const int lane = threadIdx.x;
@@ -371,7 +429,8 @@ merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ 
       }
     }
   }
-  const float inv = 1.0f / (W + exp2f(sink_log2 - M));      // the sink's term, if there is one (else exp2(-inf) = 0)
+  // the sink's term, if there is one (else exp2(-inf) = 0); sigmoid weights (plain_sum) are not normalised
+  const float inv = plain_sum ? 1.0f : 1.0f / (W + exp2f(sink_log2 - M));
 #pragma unroll
   for (int i = 0; i < DL; ++i) {
     const int d = lane + 64 * i;
@@ -390,8 +449,10 @@ static int decode_attention_launch(const void* q, long q_stride, const void* k_c
                                    float* o_part, float* lse_part, const int* block_tables, int max_blocks,
                                    const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
                                    float scale, int window, int partition, int num_splits, float sink_log2,
-                                   hipStream_t stream) {
+                                   hipStream_t stream, bool sigmoid = false, int chunk = 0, float softcap = 0.f,
+                                   const float* head_bias = nullptr) {
   if (rows <= 0) return 0;
+  if (chunk < 0 || softcap < 0.f) MIE_FAIL("decode_attention: chunk %d, score cap %g", chunk, (double)softcap);
   if (head_dim != D) MIE_FAIL("decode_attention: built for head_dim %d, called with %d", D, head_dim);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("decode_attention: %d query heads on %d kv heads", Hq, Hkv);
   if (page < 16 || page % 16) MIE_FAIL("decode_attention: page size %d (multiples of 16)", page);
@@ -406,18 +467,29 @@ static int decode_attention_launch(const void* q, long q_stride, const void* k_c
   // (the kernel writes the caches only when it is given the projection's sums)
   bf16* kc = (bf16*)const_cast<void*>(k_cache);
   bf16* vc = (bf16*)const_cast<void*>(v_cache);
-  if (num_splits == 1 && NW_WHOLE != NW_SPLIT && (long)rows * Hkv * head_tiles < NW_WHOLE_BELOW)
+  const bool whole = num_splits == 1 && NW_WHOLE != NW_SPLIT && (long)rows * Hkv * head_tiles < NW_WHOLE_BELOW;
+  if (sigmoid && whole)
+    hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, false, true>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)q, q_stride,
+                       kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
+                       scale, window, partition, num_splits, ProjectionSums{}, sink_log2, chunk, softcap, head_bias);
+  else if (sigmoid)
+    hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, false, true>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)q, q_stride,
+                       kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
+                       scale, window, partition, num_splits, ProjectionSums{}, sink_log2, chunk, softcap, head_bias);
+  else if (whole)
     hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, false>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)q, q_stride,
                        kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
-                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2);
+                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2, 0, 0.f,
+                       (const float*)nullptr);
   else
     hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, false>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)q, q_stride,
                        kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
-                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2);
+                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2, 0, 0.f,
+                       (const float*)nullptr);
   MIE_CHECK_LAUNCH("decode_attention");
   if (num_splits > 1) {
     hipLaunchKernelGGL(merge_splits_kernel, dim3(rows * Hq), dim3(64), 0, stream, o_part, lse_part, (bf16*)out, num_splits,
-                       sink_log2);
+                       sink_log2, (int)sigmoid);
     MIE_CHECK_LAUNCH("merge_splits");
   }
   return 0;
@@ -442,6 +514,19 @@ MIE_EXPORT int mie_decode_attention_sink(const void* q, long q_stride, const voi
                                  sink * 1.4426950408889634f, stream);
 }
 
+
+// Sigmoid weights instead of a softmax: a visible key counts with sigmoid(cap(score) + head_bias[head]) (head_bias
+// float32 [Hq] or null), cap(x) = softcap tanh(x / softcap) (0: none); chunk n (0: none) hides the keys before
+// floor(position / n) n.  Nothing is normalised.
+MIE_EXPORT int mie_decode_attention_sigmoid(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                            float* o_part, float* lse_part, const int* block_tables, int max_blocks,
+                                            const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
+                                            float scale, int window, int partition, int num_splits, int chunk, float softcap,
+                                            const float* head_bias, hipStream_t stream) {
+  return decode_attention_launch(q, q_stride, k_cache, v_cache, out, o_part, lse_part, block_tables, max_blocks, positions,
+                                 rows, Hq, Hkv, head_dim, page, scale, window, partition, num_splits, -INFINITY, stream, true,
+                                 chunk, softcap, head_bias);
+}
 
 // The q/k/v projection's end and the attention in one kernel, for steps whose rows and kv heads alone fill
 // the GPU (contexts unsplit).  part [splits, rows, ld] float32: the projection's sums (q heads, k heads, v
@@ -468,11 +553,13 @@ MIE_EXPORT int mie_decode_attention_from_sums(const float* part, int splits, lon
   if ((long)rows * Hkv < NW_WHOLE_BELOW)
     hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, true>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)nullptr, 0L,
                        (bf16*)k_cache, (bf16*)v_cache, (bf16*)out, (float*)nullptr, (float*)nullptr, block_tables, max_blocks,
-                       positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj, -INFINITY);
+                       positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj, -INFINITY, 0, 0.f,
+                       (const float*)nullptr);
   else
     hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, true>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)nullptr, 0L,
                        (bf16*)k_cache, (bf16*)v_cache, (bf16*)out, (float*)nullptr, (float*)nullptr, block_tables, max_blocks,
-                       positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj, -INFINITY);
+                       positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj, -INFINITY, 0, 0.f,
+                       (const float*)nullptr);
   MIE_CHECK_LAUNCH("decode_attention_from_sums");
   return 0;
 }

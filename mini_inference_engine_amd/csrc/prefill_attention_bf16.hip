@@ -26,6 +26,12 @@
 // NS - 1 - i and then stretch i: every workgroup of a row has the same number of blocks.  A block every
 // query of a wave sees whole takes a path without masks; the running maximum m is kept in units of
 // scale * log2(e); l is a per-lane partial sum, joined over a query's two lanes at the end.
+//
+// SIG: sigmoid weights instead of a softmax.  A visible key counts with sigmoid(cap(score) + the head's bias),
+// cap(x) = c tanh(x / c) or x itself, and nothing is normalised: there is no running maximum, no rescaling and
+// no denominator, the weights go straight into the second product.  A chunk size n (0: none) hides the keys
+// before floor(position / n) n.  Per score two exponentials and two reciprocals with a cap, one of each without:
+// tanh(y) = 1 - 2 / (1 + 2^(2 y log2 e)), sigmoid(z) = 1 / (1 + 2^(-z log2 e)), the constants folded.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // Waves a workgroup, at head sizes up to 128 (above, eight waves do not fit the registers: always 4):
@@ -68,13 +74,14 @@ __device__ __forceinline__ float pair_sum(float x) {
 // KS = 2: the waves form two halves that take the even and the odd 64-key blocks of the same queries (a step
 // brings 128 keys in, each half computes its 64) and join their results at the end: half the blocks a wave
 // for rows too short to give every SIMD two waves otherwise.
-template <int PF_WAVES, int KS>
+template <int PF_WAVES, int KS, bool SIG>
 __global__ void __launch_bounds__(PF_WAVES * 64)
 prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* __restrict__ k_cache,
                          const bf16* __restrict__ v_cache, bf16* __restrict__ out,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ row_start,
                          const int* __restrict__ row_position, int first_row, int Hq, int Hkv, int waves_h,
-                         int page, float scale_log2, int window, float sink_log2) {
+                         int page, float scale_log2, int window, float sink_log2, int chunk, float softcap,
+                         const float* __restrict__ head_bias) {
   extern __shared__ __align__(16) unsigned char pf_lds[];
   constexpr int PF_THREADS = PF_WAVES * 64;
   constexpr int SUB_WAVES = PF_WAVES / KS;                   // waves of one half
@@ -153,11 +160,33 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
     }
     // keys the wave's queries can see, and the workgroup's (the union over its waves)
     const int wave_kmax = tile_ok ? tile_last : -1;            // -1: the wave has no query
-    const int wave_kmin = window > 0 ? tile_first - window + 1 : 0;
+    int wave_kmin = window > 0 ? tile_first - window + 1 : 0;
     const int end_q = (s + 1) * STRETCH < q_len ? (s + 1) * STRETCH : q_len;
     const int kmax = p0 + end_q - 1;
     int kmin = window > 0 ? p0 + s * STRETCH - window + 1 : 0;
     kmin = kmin > 0 ? kmin : 0;
+    int q_lo = 0, tile_lo = 0;                                 // SIG: first key of the lane's query's chunk, of the tile's last query's
+    float sg_c1 = 0.f, sg_c2 = 0.f, sg_c3 = 0.f;
+    if constexpr (SIG) {
+      if (chunk > 0) {
+        const int c_wave = tile_first / chunk * chunk, c_str = (p0 + s * STRETCH) / chunk * chunk;
+        wave_kmin = wave_kmin > c_wave ? wave_kmin : c_wave;
+        kmin = kmin > c_str ? kmin : c_str;
+        q_lo = qpos / chunk * chunk;
+        tile_lo = tile_last / chunk * chunk;
+      }
+      // here scale_log2 carries the plain scale
+      const float hb = head_bias ? head_bias[head] : 0.f;
+      const float L2E = 1.4426950408889634f;
+      if (softcap > 0.f) {
+        sg_c1 = 2.f * L2E * scale_log2 / softcap;
+        sg_c2 = 2.f * L2E * softcap;
+        sg_c3 = -L2E * (softcap + hb);
+      } else {
+        sg_c1 = -L2E * scale_log2;
+        sg_c3 = -L2E * hb;
+      }
+    }
     const int blk0 = kmin & ~(PF_BK - 1);
     const int last_blk = kmax & ~(PF_BK - 1);
 
@@ -283,7 +312,50 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
         }
       }
       // every query of the tile sees every key of the block (uniform over the wave)
-      const bool whole = blk + PF_BK - 1 <= tile_first && (window <= 0 || blk >= tile_last - window + 1);
+      const bool whole = blk + PF_BK - 1 <= tile_first && (window <= 0 || blk >= tile_last - window + 1) &&
+                         (!SIG || blk >= tile_lo);
+      if constexpr (SIG) {
+        if (softcap > 0.f) {
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const float r = __builtin_amdgcn_rcpf(1.f + fast_exp2(S[u][i] * sg_c1));
+              S[u][i] = __builtin_amdgcn_rcpf(1.f + fast_exp2(fmaf(r, sg_c2, sg_c3)));
+            }
+        } else {
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[u][i] = __builtin_amdgcn_rcpf(1.f + fast_exp2(fmaf(S[u][i], sg_c1, sg_c3)));
+        }
+        if (!whole) {
+          const int hi = tile_ok ? qpos : -1;                  // a tile that does not exist sees nothing
+          int lo = window > 0 ? hi - window + 1 : 0;
+          lo = lo > q_lo ? lo : q_lo;
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int key = blk + 32 * u + 8 * (i >> 2) + 4 * g + (i & 3);
+              S[u][i] = key >= lo && key <= hi ? S[u][i] : 0.f;
+            }
+        }
+        Frag pb[4];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pb[2 * u + (e >> 2)].w[e & 3] = pack_bf16(S[u][2 * e], S[u][2 * e + 1]);
+#pragma unroll
+        for (int dt = 0; dt < DT32; ++dt)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            Frag va;
+            va.q = *reinterpret_cast<const uint4*>(Vb + dt * 32 * PF_VROW + t * 32);
+            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va.v, pb[t].v, O[dt], 0, 0, 0);
+          }
+        return;
+      }
       float alpha;
       if (whole) {
         float mx[4];
@@ -402,7 +474,14 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
           for (int i = 0; i < 16; ++i) xch[64 * (2 + dt * 16 + i)] = O[dt][i];
       }
       __syncthreads();
-      if (wk == 0) {
+      if (SIG) {
+        if (wk == 0) {
+#pragma unroll
+          for (int dt = 0; dt < DT32; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) O[dt][i] += xch[64 * (2 + dt * 16 + i)];
+        }
+      } else if (wk == 0) {
         const float m1 = xch[0], l1 = xch[64];
         const float mj = max_nn(m, m1);
         // a half may have seen no key of a query (m = -inf, sums 0): it counts for nothing
@@ -420,7 +499,7 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
     const float total = pair_sum(l);
     if (q_ok && wk == 0) {
       // a sink (sink_log2 > -inf) is one more term in the denominator; m is finite: a query sees its own key
-      const float inv = 1.0f / (total + fast_exp2(sink_log2 - m));
+      const float inv = SIG ? 1.0f : 1.0f / (total + fast_exp2(sink_log2 - m));
       bf16* op = out + ((size_t)qtok * Hq + head) * D + 4 * g;
 #pragma unroll
       for (int dt = 0; dt < DT32; ++dt)
@@ -446,8 +525,10 @@ static int prefill_attention_launch(const void* q, long q_stride, const void* k_
                                     const int* block_tables, int max_blocks, const int* row_start,
                                     const int* row_position, int first_row, int rows, int max_row_tokens, int Hq,
                                     int Hkv, int head_dim, int page, float scale, int window, float sink_log2,
-                                    hipStream_t stream) {
+                                    hipStream_t stream, bool sigmoid = false, int chunk = 0, float softcap = 0.f,
+                                    const float* head_bias = nullptr) {
   if (rows <= 0 || max_row_tokens <= 0) return 0;
+  if (chunk < 0 || softcap < 0.f) MIE_FAIL("prefill_attention: chunk %d, score cap %g", chunk, (double)softcap);
   if (head_dim != D) MIE_FAIL("prefill_attention: built for head_dim %d, called with %d", D, head_dim);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("prefill_attention: %d query heads on %d kv heads", Hq, Hkv);
   if (page < 16 || page % 16) MIE_FAIL("prefill_attention: page size %d (multiples of 16)", page);
@@ -489,26 +570,30 @@ static int prefill_attention_launch(const void* q, long q_stride, const void* k_
   }
   plan(kind == EIGHT_QUERIES ? 8 : 4, &waves_h, &grid);
   if (grid.y > 65535 || grid.z > 65535) MIE_FAIL("prefill_attention: grid too large (%d rows)", rows);
-  const float scale_log2 = scale * 1.4426950408889634f;
+  const float scale_log2 = sigmoid ? scale : scale * 1.4426950408889634f;      // the sigmoid kernels fold their own constants
   // more LDS than a kernel gets by default is asked for once per kernel and device
-  static bool lds_allowed[3][64] = {};
+  static bool lds_allowed[6][64] = {};
   auto launch = [&](auto kernel, int waves, int lds_bytes) -> int {
-    if (lds_bytes > 64 * 1024 && !lds_allowed[kind][dev]) {
+    const int which = kind + (sigmoid ? 3 : 0);
+    if (lds_bytes > 64 * 1024 && !lds_allowed[which][dev]) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
       if (e != hipSuccess) MIE_FAIL("prefill_attention: %d bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
-      lds_allowed[kind][dev] = true;
+      lds_allowed[which][dev] = true;
     }
     hipLaunchKernelGGL(kernel, grid, dim3(waves * 64), lds_bytes, stream, (const bf16*)q, q_stride, (const bf16*)k_cache,
                        (const bf16*)v_cache, (bf16*)out, block_tables, max_blocks, row_start, row_position, first_row, Hq, Hkv,
-                       waves_h, page, scale_log2, window, sink_log2);
+                       waves_h, page, scale_log2, window, sink_log2, chunk, softcap, head_bias);
     return 0;
   };
   int rc = 0;
   if constexpr (PF_MAX_WAVES == 8) {
-    if (kind == EIGHT_QUERIES) rc = launch(prefill_attention_kernel<8, 1>, 8, 2 * PF_BUF);
-    if (kind == EIGHT_KEYS) rc = launch(prefill_attention_kernel<8, 2>, 8, 4 * PF_BUF);
+    if (kind == EIGHT_QUERIES && !sigmoid) rc = launch(prefill_attention_kernel<8, 1, false>, 8, 2 * PF_BUF);
+    if (kind == EIGHT_KEYS && !sigmoid) rc = launch(prefill_attention_kernel<8, 2, false>, 8, 4 * PF_BUF);
+    if (kind == EIGHT_QUERIES && sigmoid) rc = launch(prefill_attention_kernel<8, 1, true>, 8, 2 * PF_BUF);
+    if (kind == EIGHT_KEYS && sigmoid) rc = launch(prefill_attention_kernel<8, 2, true>, 8, 4 * PF_BUF);
   }
-  if (kind == FOUR) rc = launch(prefill_attention_kernel<4, 1>, 4, 2 * PF_BUF);
+  if (kind == FOUR && !sigmoid) rc = launch(prefill_attention_kernel<4, 1, false>, 4, 2 * PF_BUF);
+  if (kind == FOUR && sigmoid) rc = launch(prefill_attention_kernel<4, 1, true>, 4, 2 * PF_BUF);
   if (rc) return rc;
   MIE_CHECK_LAUNCH("prefill_attention");
   return 0;
@@ -531,4 +616,17 @@ MIE_EXPORT int mie_prefill_attention_sink(const void* q, long q_stride, const vo
   return prefill_attention_launch(q, q_stride, k_cache, v_cache, out, block_tables, max_blocks, row_start, row_position,
                                   first_row, rows, max_row_tokens, Hq, Hkv, head_dim, page, scale, window,
                                   sink * 1.4426950408889634f, stream);
+}
+
+// Sigmoid weights instead of a softmax: a visible key counts with sigmoid(cap(score) + head_bias[head]) (head_bias
+// float32 [Hq] or null), cap(x) = softcap tanh(x / softcap) (0: none); chunk n (0: none) hides the keys before
+// floor(position / n) n.  Nothing is normalised.
+MIE_EXPORT int mie_prefill_attention_sigmoid(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                             const int* block_tables, int max_blocks, const int* row_start,
+                                             const int* row_position, int first_row, int rows, int max_row_tokens, int Hq,
+                                             int Hkv, int head_dim, int page, float scale, int window, int chunk,
+                                             float softcap, const float* head_bias, hipStream_t stream) {
+  return prefill_attention_launch(q, q_stride, k_cache, v_cache, out, block_tables, max_blocks, row_start, row_position,
+                                  first_row, rows, max_row_tokens, Hq, Hkv, head_dim, page, scale, window, -INFINITY, stream,
+                                  true, chunk, softcap, head_bias);
 }

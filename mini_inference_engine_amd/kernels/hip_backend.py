@@ -1111,15 +1111,15 @@ class HipBackend(KernelBackend):
         done = 0
         if D > 256:
             force_generic = True            # beyond the matrix-core kernels' head sizes: the 32-bit kernel takes up to 1,024
-        if sigmoid:
-            force_generic = True
         if qkv.dtype == torch.bfloat16 and not force_generic and step.num_decode_rows > 0:
             done = step.num_decode_rows        # single-token rows lead the batch: token t is row t
             lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))
             block_keys = lib.mie_decode_block_keys()
-            partition, splits = self.decode_splits(done, Hq, Hkv, step.max_context, window, block_keys, D)
+            # a row sees at most a chunk's keys: the splits are planned as for a window of that many
+            reach = min(window or chunk, chunk or window) if (window or chunk) else None
+            partition, splits = self.decode_splits(done, Hq, Hkv, step.max_context, reach, block_keys, D)
             if num_splits is not None:
-                bound = min(step.max_context, window + 32) if window else step.max_context
+                bound = min(step.max_context, reach + 32) if reach else step.max_context
                 partition = -(-(-(-bound // num_splits)) // block_keys) * block_keys
                 splits = max(1, -(-bound // partition))
             o_part = lse_part = None
@@ -1129,11 +1129,15 @@ class HipBackend(KernelBackend):
             args = (_ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(o_part), _ptr(lse_part),
                     _ptr(bt), bt.shape[1], _ptr(step.positions), done, Hq, Hkv, D, page, float(scale), int(window or 0),
                     partition, splits)
-            if has_sink:
+            if sigmoid:
+                library.check(lib, lib.mie_decode_attention_sigmoid(*args, int(chunk or 0), float(softcap or 0.0),
+                                                                    _ptr(head_bias), self._stream()))
+            elif has_sink:
                 library.check(lib, lib.mie_decode_attention_sink(*args, sink, self._stream()))
             else:
                 library.check(lib, lib.mie_decode_attention(*args, self._stream()))
-        if done < T and qkv.dtype == torch.bfloat16 and not force_generic:
+        end = T                                # tokens [done, end) are left to the 32-bit kernel
+        if step.num_decode_rows < T and qkv.dtype == torch.bfloat16 and not force_generic:
             # rows of several tokens: matrix-core kernel over their own and earlier portions' keys
             for name, t, n in (("row_start", step.row_start, step.num_rows + 1),
                                ("row_position", step.row_position, step.num_rows)):
@@ -1144,18 +1148,21 @@ class HipBackend(KernelBackend):
                     _ptr(step.row_start), _ptr(step.row_position), step.num_decode_rows,
                     step.num_rows - step.num_decode_rows, step.max_row_tokens, Hq, Hkv, D, page, float(scale),
                     int(window or 0))
-            if has_sink:
+            if sigmoid:
+                library.check(lib, lib.mie_prefill_attention_sigmoid(*args, int(chunk or 0), float(softcap or 0.0),
+                                                                     _ptr(head_bias), self._stream()))
+            elif has_sink:
                 library.check(lib, lib.mie_prefill_attention_sink(*args, sink, self._stream()))
             else:
                 library.check(lib, lib.mie_prefill_attention(*args, self._stream()))
-            done = T
-        if done < T:
+            end = step.num_decode_rows
+        if done < end:
             lib = self.lib("attention")
             esz = qkv.element_size()
             args = (c_void_p(qkv.data_ptr() + done * qkv.stride(0) * esz), qkv.stride(0), _ptr(k_cache), _ptr(v_cache),
                     c_void_p(out.data_ptr() + done * Hq * D * esz), _code(qkv.dtype), _ptr(bt), bt.shape[1],
                     c_void_p(step.token_row.data_ptr() + done * 4), c_void_p(step.positions.data_ptr() + done * 4),
-                    T - done, Hq, Hkv, D, page, float(scale), int(window or 0), has_sink, sink)
+                    end - done, Hq, Hkv, D, page, float(scale), int(window or 0), has_sink, sink)
             if scored:
                 library.check(lib, lib.mie_paged_attention_scored(*args, int(chunk or 0), float(softcap or 0.0), int(sigmoid),
                                                                   _ptr(head_bias), self._stream()))

@@ -570,6 +570,8 @@ class AttentionCase:
         self.step = SimpleNamespace(token_row=self.token_row, positions=self.positions, num_tokens=self.num_tokens,
                                     num_rows=len(rows), num_decode_rows=self.num_decode_rows,
                                     row_start=torch.tensor(rs, dtype=torch.int32).cuda(), host={"row_start": rs},
+                                    row_position=torch.tensor([h for h, _ in rows], dtype=torch.int32).cuda(),
+                                    max_row_tokens=max(n for _, n in rows),
                                     groups=[self.group], max_context=max(h + n for h, n in rows))
 
 
