@@ -27,6 +27,9 @@ struct GroupedArgs {
   const int* gather; int gather_div;
   int M, N, K, G, act;
   const void* zeros;            // 64 bytes of zeros in device memory: what a load beyond a tile's rows or beyond K reads
+  // glu != 0 (matrix-core kernel only): W's rows alternate in blocks of 16 gate rows and 16 up rows, and C [.., N / 2]
+  // receives g * sigmoid(glu_alpha g) * (u + 1), g = min(gate sum, glu_limit), u = clamp(up sum, -glu_limit, glu_limit)
+  int glu; float glu_limit, glu_alpha;
 };
 
 template <typename TA, typename TW, typename TC>
@@ -294,6 +297,25 @@ grouped_gemm_ring_kernel(GroupedArgs p) {
   GG_VMCNT(0);                         // nothing of this wave may still be writing the LDS when it ends
   const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * (TN / 2);
   TC* C = (TC*)p.C + (size_t)g * p.c_group;
+  if (p.glu) {
+    // tiles 2 jj and 2 jj + 1 of a lane are the gate and the up sums of the same 16 inner channels
+#pragma unroll
+    for (int jj = 0; jj < NT / 2; ++jj) {
+      if (n0 + wn + (2 * jj + 1) * 16 + col >= p.N) continue;
+      const int n = (n0 + wn) / 2 + jj * 16 + col;
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int m = m0 + wm + i * 16 + kb * 4 + e;
+          if (m >= m_end) continue;
+          const float gt = fminf(acc[i][2 * jj][e], p.glu_limit);
+          const float up = fminf(fmaxf(acc[i][2 * jj + 1][e], -p.glu_limit), p.glu_limit);
+          C[(size_t)(c_row0 + m) * p.ldc + n] = from_float<TC>(gt * mie_sigmoid(p.glu_alpha * gt) * (up + 1.0f));
+        }
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
     const int n = n0 + wn + j * 16 + col;
@@ -339,19 +361,22 @@ static int launch_grouped(const GroupedArgs& p, int c_dtype, dim3 grid, hipStrea
 // Strides and group offsets are in elements.  zeros: 64 bytes of zeros in device memory (or null: the kernels that
 // need them are not used).  Rows shape: offs non-null, M = the length of the sorted list (an upper
 // bound of any group's rows), a_group / c_group / a_mod unused.
-MIE_EXPORT int mie_grouped_linear(const void* A, int a_dtype, long lda, long a_group, int a_mod, const void* W, int w_dtype,
-                                  long ldw, long w_group, void* C, int c_dtype, long ldc, long c_group, const float* bias,
-                                  const float* gate, long ldg, const int* offs, const int* gather, int gather_div, int M,
-                                  int N, int K, int G, int act, const void* zeros, hipStream_t s) {
+static int grouped_linear_run(const void* A, int a_dtype, long lda, long a_group, int a_mod, const void* W, int w_dtype,
+                              long ldw, long w_group, void* C, int c_dtype, long ldc, long c_group, const float* bias,
+                              const float* gate, long ldg, const int* offs, const int* gather, int gather_div, int M,
+                              int N, int K, int G, int act, const void* zeros, int glu, float glu_limit, float glu_alpha,
+                              hipStream_t s) {
   if (M <= 0 || N <= 0 || G <= 0) return 0;
   if (K <= 0 || !A || !W || !C) MIE_FAIL("grouped_linear: K %d or a null operand", K);
   if (lda < K && !offs && a_group == 0) MIE_FAIL("grouped_linear: A row stride %ld < K %d", lda, K);
-  if (ldw < K || ldc < N) MIE_FAIL("grouped_linear: strides %ld, %ld for K %d, N %d", ldw, ldc, K, N);
+  if (ldw < K || ldc < (glu ? N / 2 : N)) MIE_FAIL("grouped_linear: strides %ld, %ld for K %d, N %d", ldw, ldc, K, N);
+  if (glu && (N % 32 || bias || gate || !(glu_limit > 0.f)))
+    MIE_FAIL("grouped_linear: the gated epilogue takes N %d in blocks of 16 gate and 16 up rows, no bias, limit %g", N, (double)glu_limit);
   if (a_mod <= 0) a_mod = G;
   if (gather && gather_div <= 0) MIE_FAIL("grouped_linear: gather divisor %d", gather_div);
   if (act < MIE_ACT_NONE || act > MIE_ACT_RELU2) MIE_FAIL("grouped_linear: activation code %d", act);
   GroupedArgs p = {A, lda, offs ? 0 : a_group, offs ? 1 : a_mod, W, ldw, w_group, C, ldc, offs ? 0 : c_group, bias, gate, ldg,
-                   offs, gather, gather_div, M, N, K, G, act, zeros};
+                   offs, gather, gather_div, M, N, K, G, act, zeros, glu, glu_limit, glu_alpha};
   const long mt = (M + GG_T - 1) / GG_T + (offs ? G : 0);
   if (mt > 65535 || G > 65535) MIE_FAIL("grouped_linear: %ld row tiles, %d groups are beyond the grid", mt, G);
   dim3 grid((N + GG_T - 1) / GG_T, (unsigned)mt, offs ? 1 : G);
@@ -373,11 +398,31 @@ MIE_EXPORT int mie_grouped_linear(const void* A, int a_dtype, long lda, long a_g
     MIE_CHECK_LAUNCH("grouped_linear");
     return 0;
   }
+  if (glu) MIE_FAIL("grouped_linear: the gated epilogue needs bfloat16 operands with K %d, strides %ld, %ld multiples of 8", K, lda, ldw);
   if (a_dtype == MIE_F32 && w_dtype == MIE_F32) return launch_grouped<float, float>(p, c_dtype, grid, s);
   if (a_dtype == MIE_F32 && w_dtype == MIE_BF16) return launch_grouped<float, bf16>(p, c_dtype, grid, s);
   if (a_dtype == MIE_BF16 && w_dtype == MIE_F32) return launch_grouped<bf16, float>(p, c_dtype, grid, s);
   if (a_dtype == MIE_BF16 && w_dtype == MIE_BF16) return launch_grouped<bf16, bf16>(p, c_dtype, grid, s);
   MIE_FAIL("grouped_linear: dtype codes A %d, W %d", a_dtype, w_dtype);
+}
+
+MIE_EXPORT int mie_grouped_linear(const void* A, int a_dtype, long lda, long a_group, int a_mod, const void* W, int w_dtype,
+                                  long ldw, long w_group, void* C, int c_dtype, long ldc, long c_group, const float* bias,
+                                  const float* gate, long ldg, const int* offs, const int* gather, int gather_div, int M,
+                                  int N, int K, int G, int act, const void* zeros, hipStream_t s) {
+  return grouped_linear_run(A, a_dtype, lda, a_group, a_mod, W, w_dtype, ldw, w_group, C, c_dtype, ldc, c_group, bias, gate, ldg,
+                            offs, gather, gather_div, M, N, K, G, act, zeros, 0, 0.f, 0.f, s);
+}
+
+// The same in the rows shape for gated experts, on the matrix cores only (bfloat16 A and W, K and the strides multiples
+// of 8): W's N rows alternate in blocks of 16 gate rows and 16 up rows, C [rows, N / 2] receives
+// g * sigmoid(alpha g) * (u + 1) with g = min(gate sum, limit), u = clamp(up sum, -limit, limit).
+MIE_EXPORT int mie_grouped_glu(const void* A, int a_dtype, long lda, const void* W, int w_dtype, long ldw, long w_group, void* C,
+                               int c_dtype, long ldc, const int* offs, const int* gather, int gather_div, int M, int N, int K,
+                               int G, float limit, float alpha, const void* zeros, hipStream_t s) {
+  if (!offs || !zeros) MIE_FAIL("grouped_glu: group offsets and the block of zeros are needed");
+  return grouped_linear_run(A, a_dtype, lda, 0, 1, W, w_dtype, ldw, w_group, C, c_dtype, ldc, 0, nullptr, nullptr, 0, offs, gather,
+                            gather_div, M, N, K, G, MIE_ACT_NONE, zeros, 1, limit, alpha, s);
 }
 
 // ---- router, one thread a token.  over_all == 0: the `top` largest of logits[t, :] + bias (lowest index first among
@@ -429,13 +474,65 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, long ld, con
   }
 }
 
+// The same with a token's values kept in the LDS (up to ROUTE_LDS_E router outputs): every logit is read once and
+// every exponential taken once; a chosen output is struck out where it stands.  Same sums in the same order, same
+// choices.
+#define ROUTE_LDS_E 128
+__global__ void __launch_bounds__(64)
+route_topk_lds_kernel(const float* __restrict__ logits, long ld, const float* __restrict__ bias,
+                      const float* __restrict__ choice_bias, int over_all, int* __restrict__ experts,
+                      float* __restrict__ shares, int T, int E, int top) {
+  __shared__ float sc[ROUTE_LDS_E * 64];
+  const int t = blockIdx.x * 64 + threadIdx.x;
+  if (t >= T) return;
+  float* mine = sc + threadIdx.x;            // value e at mine[64 e]: a bank a thread
+  const float* z = logits + (size_t)t * ld;
+  float largest = -INFINITY;
+  for (int e = 0; e < E; ++e) {
+    const float v = z[e] + (bias ? bias[e] : 0.f);
+    mine[64 * e] = v;
+    largest = fmaxf(largest, v);
+  }
+  if (over_all) {
+    float total = 0.f;
+    for (int e = 0; e < E; ++e) total += expf(mine[64 * e] - largest);
+    for (int e = 0; e < E; ++e) mine[64 * e] = expf(mine[64 * e] - largest) / total;
+  }
+  int* ex = experts + (size_t)t * top;
+  float* sh = shares + (size_t)t * top;
+  for (int j = 0; j < top; ++j) {
+    int best = -1;
+    float bv = 0.f, bs = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const float s = mine[64 * e];
+      if (s == -INFINITY) continue;            // struck out
+      const float v = over_all && choice_bias ? s + choice_bias[e] : s;
+      if (best < 0 || v > bv) { best = e; bv = v; bs = s; }
+    }
+    if (best < 0) best = 0;                    // every value left is -inf: cannot happen with finite logits
+    ex[j] = best;
+    sh[j] = bs;
+    mine[64 * best] = -INFINITY;
+  }
+  if (!over_all) {
+    float sum = 0.f;
+    const float first = sh[0];
+    for (int j = 0; j < top; ++j) sum += expf(sh[j] - first);
+    for (int j = 0; j < top; ++j) sh[j] = expf(sh[j] - first) / sum;
+  }
+}
+
 static int route_topk_launch(const float* logits, long ld, const float* bias, const float* choice_bias, int over_all,
                              int* experts, float* shares, int T, int E, int top, hipStream_t s) {
   if (T <= 0) return 0;
   if (E <= 0 || top <= 0 || top > E || top > ROUTE_MAX_TOP) MIE_FAIL("route_topk: top %d of %d experts (at most %d)", top, E, ROUTE_MAX_TOP);
   if (ld < E) MIE_FAIL("route_topk: row stride %ld < %d", ld, E);
-  hipLaunchKernelGGL(route_topk_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, ld, bias, choice_bias, over_all, experts,
-                     shares, T, E, top);
+  if (E <= ROUTE_LDS_E)
+    hipLaunchKernelGGL(route_topk_lds_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, ld, bias, choice_bias, over_all,
+                       experts, shares, T, E, top);
+  else
+    hipLaunchKernelGGL(route_topk_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, ld, bias, choice_bias, over_all, experts,
+                       shares, T, E, top);
   MIE_CHECK_LAUNCH("route_topk");
   return 0;
 }

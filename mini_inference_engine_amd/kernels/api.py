@@ -172,10 +172,18 @@ class KernelBackend:
         -> (experts [T, top] int32, shares [T, top] float32)."""
         raise NotImplementedError
 
-    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None):
+    def glu_rows_block(self, inner: int) -> int:
+        """How ``routed_experts`` wants a gated expert's 2 * inner stacked rows: 0, the gate rows before the up rows; n
+        (a divisor of inner), alternating blocks of n gate rows and n up rows (the kernels then meet a channel's gate
+        and up sums in one place).  A part asks once, orders its rows so and passes the answer on as ``glu_block``."""
+        return 0
+
+    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None,
+                       glu_block=0):
         """y[t] = sum_j shares[t, j] * W_down[e] act(W_up[e] x[t]), e = experts[t, j]; w_up [E, ff, width],
         w_down [E, width, ff]; the hidden activation is rounded once to the activation dtype -> [T, width] float32.
-        ``gated`` = (limit, alpha): w_up is [E, 2 ff, width], an expert's gate rows before its up rows, and the hidden
+        ``gated`` = (limit, alpha): w_up is [E, 2 ff, width], an expert's gate rows before its up rows (or in
+        alternating blocks of ``glu_block`` gate rows and as many up rows: see glu_rows_block), and the hidden
         activation is g * sigmoid(alpha g) * (u + 1) with g = min(gate sum, limit), u = clamp(up sum, -limit, limit),
         ``activation`` unused.  ``identity_from`` = E: a choice e >= E is an expert that returns x[t] itself (such
         choices may be all there are: w_up and w_down None)."""

@@ -669,7 +669,13 @@ class HipBackend(KernelBackend):
                                               self._stream()))
         return experts, shares
 
-    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None):
+    GLU_BLOCK = 16      # the matrix-core kernel's tiles are 16 columns wide: a lane holds columns c and c + 16 of its row
+
+    def glu_rows_block(self, inner):
+        return self.GLU_BLOCK if self.act_dtype == torch.bfloat16 and inner % self.GLU_BLOCK == 0 else 0
+
+    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None,
+                       glu_block=0):
         self._on_device(x, experts, shares, w_up, w_down)
         _rows_ok(x, "routed_experts: x")
         T, W = x.shape
@@ -708,7 +714,19 @@ class HipBackend(KernelBackend):
         if gated is None:
             self._grouped(x, x.stride(0), 0, 1, w_up, W, ff * W, hidden, ff, 0, n, ff, W, E, offs=offs, gather=order,
                           gather_div=top, act=activation)
+        elif (glu_block == self.GLU_BLOCK and x.dtype == torch.bfloat16 and w_up.dtype == torch.bfloat16 and W % 8 == 0
+              and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w_up.data_ptr() % 16 == 0):
+            # gate and up sums meet in the product's own epilogue: the hidden activation is written once, rounded once
+            if self._zeros is None:
+                self._zeros = torch.zeros(64, dtype=torch.int32, device=dev)
+            limit, alpha = gated
+            library.check(lib, lib.mie_grouped_glu(_ptr(x), _code(x.dtype), x.stride(0), _ptr(w_up), _code(w_up.dtype), W,
+                                                   2 * ff * W, _ptr(hidden), _code(hidden.dtype), ff, _ptr(offs), _ptr(order),
+                                                   top, n, 2 * ff, W, E, float(limit), float(alpha), _ptr(self._zeros),
+                                                   self._stream()))
         else:
+            if glu_block and ff % glu_block:
+                raise ValueError(f"routed_experts: blocks of {glu_block} rows in experts of inner size {ff}")
             limit, alpha = gated
             gu = torch.empty((n, 2 * ff), dtype=torch.float32, device=dev)
             self._grouped(x, x.stride(0), 0, 1, w_up, W, 2 * ff * W, gu, 2 * ff, 0, n, 2 * ff, W, E, offs=offs, gather=order,
@@ -716,7 +734,7 @@ class HipBackend(KernelBackend):
             glib = self.lib("gemm")
             # rows of identity choices hold whatever was there: the function of it is never read
             library.check(glib, glib.mie_clamped_glu(_ptr(gu), gu.stride(0), _ptr(hidden), hidden.stride(0), _code(hidden.dtype),
-                                                     n, ff, float(limit), float(alpha), self._stream()))
+                                                     n, ff, float(limit), float(alpha), int(glu_block), self._stream()))
         y = torch.empty((n, W), dtype=torch.float32, device=dev)
         self._grouped(hidden, ff, 0, 1, w_down, ff, W * ff, y, W, 0, n, W, ff, E, offs=offs)
         if identity_from is None:

@@ -27,10 +27,11 @@ register_kernel_module("gemm", {
     "mie_silu_mul": [P, L, P, L, I, I, I, P],
     "mie_act_mul": [P, L, P, L, I, I, I, I, P],
     "mie_act_store": [P, L, P, L, I, I, I, I, P],
-    "mie_clamped_glu": [P, L, P, L, I, I, I, F, F, P],
+    "mie_clamped_glu": [P, L, P, L, I, I, I, F, F, I, P],
 })
 register_kernel_module("grouped_gemm", {
     "mie_grouped_linear": [P, I, L, L, I, P, I, L, L, P, I, L, L, P, P, L, P, P, I, I, I, I, I, I, P, P],
+    "mie_grouped_glu": [P, I, L, P, I, L, L, P, I, L, P, P, I, I, I, I, I, F, F, P, P],
     "mie_route_topk": [P, L, P, P, P, I, I, I, P],
     "mie_route_topk_all": [P, L, P, P, P, P, I, I, I, P],
     "mie_moe_align": [P, I, I, P, P, P, P],

@@ -58,10 +58,18 @@ class RoutedExperts(FeedForward):
         return specs
 
     def prepare(self, device, dtype):
+        first = not getattr(self, "_prepared", False)
+        self._prepared = True
         for attr in ("b_router", "choice_bias"):        # router logits and scores are 32-bit
             t = getattr(self, attr, None)
             if t is not None:
                 setattr(self, attr, t.float().contiguous())
+        if first and self.gated is not None and self.num_experts:
+            # the kernels may want a channel's gate row and up row near each other: blocks of n gate rows, n up rows
+            self.glu_block = n = int(self.ops.glu_rows_block(self.inner))
+            if n:
+                E, f, w = self.num_experts, self.inner, self.width
+                self.w_up = self.w_up.view(E, 2, f // n, n, w).transpose(1, 2).contiguous().view(E * 2 * f, w)
 
     def forward(self, x, step, add_to=None):
         import torch
@@ -72,5 +80,8 @@ class RoutedExperts(FeedForward):
         rows = self.inner if self.gated is None else 2 * self.inner
         w_up = None if not E else self.w_up.view(E, rows, self.width)
         w_down = None if not E else self.w_down.view(E, self.width, self.inner)
+        if self.gated is None or not getattr(self, "glu_block", 0):
+            return ops.routed_experts(x, experts, shares, w_up, w_down, self.activation, gated=self.gated,
+                                      identity_from=E if self.identity else None)
         return ops.routed_experts(x, experts, shares, w_up, w_down, self.activation, gated=self.gated,
-                                  identity_from=E if self.identity else None)
+                                  identity_from=E if self.identity else None, glu_block=self.glu_block)

@@ -662,7 +662,8 @@ def test_norm_per_head_and_store_kernel(hip, dtype):
 def test_routing_over_all_outputs_and_gated_expert_kernels(hip, dtype):
     ops, g = hip[dtype], torch.Generator().manual_seed(14)
     for (T, W, E, I, top, ff, limit) in ((1, 64, 5, 2, 3, 48, 1.5), (37, 48, 4, 1, 5, 24, 3.0), (300, 72, 3, 0, 1, 40, 0.8),
-                                         (9, 64, 0, 3, 2, 8, 1.0), (130, 128, 16, 2, 4, 96, 7.0), (65, 70, 2, 2, 2, 18, 0.5)):
+                                         (9, 64, 0, 3, 2, 8, 1.0), (130, 128, 16, 2, 4, 96, 7.0), (65, 70, 2, 2, 2, 18, 0.5),
+                                         (700, 64, 4, 1, 2, 64, 2.0), (2, 256, 8, 0, 2, 160, 1.0)):
         R = E + I
         logits, corr = _rand((T, R), torch.float32, g, 2.0), _rand((R,), torch.float32, g, 0.25)
         idx, shares = ops.route_topk(logits, None, top, over="all", choice_bias=corr)
@@ -677,6 +678,13 @@ def test_routing_over_all_outputs_and_gated_expert_kernels(hip, dtype):
         got = ops.routed_experts(x, idx, shares, w_up, w_down, "relu2", gated=(limit, 1.702), identity_from=E if I else None)
         want = ref.ref_routed_experts(x, idx, shares, w_up, w_down, "relu2", dtype, gated=(limit, 1.702), identity_from=E if I else None)
         close(got, want, 1e-5 if dtype == torch.float32 else 1e-2, f"experts {T} tokens, {E}+{I} outputs")
+        if E and ff % 16 == 0:
+            # rows in alternating blocks of 16 gate and 16 up rows: in bfloat16 the product's own epilogue gates
+            assert ops.glu_rows_block(ff) == (16 if dtype == torch.bfloat16 else 0)
+            mixed = w_up.view(E, 2, ff // 16, 16, W).transpose(1, 2).contiguous().view(E, 2 * ff, W)
+            got = ops.routed_experts(x, idx, shares, mixed, w_down, "relu2", gated=(limit, 1.702),
+                                     identity_from=E if I else None, glu_block=16)
+            close(got, want, 1e-5 if dtype == torch.float32 else 1e-2, f"experts in blocks of 16, {T} tokens")
     tie = torch.zeros(2, 4).cuda()
     assert ops.route_topk(tie, None, 2, over="all")[0].tolist() == [[0, 1], [0, 1]], "lowest index first among equals"
     moved = ops.route_topk(tie, None, 2, over="all", choice_bias=torch.tensor([0.0, 0.0, 0.5, 0.25]).cuda())

@@ -432,7 +432,8 @@ class TorchBackend(KernelBackend):
     def route_topk(self, logits, bias, top, over="chosen", choice_bias=None):
         return ref_route_topk(logits, bias, top, over, choice_bias)
 
-    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None):
+    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None, glu_block=0):
+        assert glu_block == 0, "the torch operations keep gate rows before up rows"
         self._count("routed_experts")
         return ref_routed_experts(x, experts, shares, w_up, w_down, activation, self.act_dtype, gated, identity_from)
 
