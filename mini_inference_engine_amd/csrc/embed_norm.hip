@@ -617,6 +617,108 @@ MIE_EXPORT int mie_norm_pair_conv(const float* stream, const float* w1, const fl
   return 0;
 }
 
+// ---- a normed branch output added to the stream, and the next sublayer's normed, convolved input, for steps whose rows
+// are single tokens (every input before a row's token comes from its tail):
+//   stream[t] += y[t] * rstd(y[t]) * wb;  h = stream[t] * rstd(stream[t]) * w1;
+//   xm[t] = h + sum_k taps[:, k] * (k == K - 1 ? h : tail[slot][k]);  tail[slot] moves on by h.
+// One workgroup a token; widths that are a multiple of 4 up to 8192; the sums in the order of the two kernels it replaces.
+template <typename TO, int K>
+__global__ void __launch_bounds__(NORM_THREADS)
+branch_norm_conv_single_kernel(const float* __restrict__ y, float* __restrict__ stream, const float* __restrict__ wb, float eps_b,
+                               const float* __restrict__ w1, const float* __restrict__ taps, float* __restrict__ tail,
+                               const int* __restrict__ slots, TO* __restrict__ xm, int width, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, nv = width / 4;
+  const float4* yr = reinterpret_cast<const float4*>(y + (size_t)t * width);
+  float4* sr = reinterpret_cast<float4*>(stream + (size_t)t * width);
+  float4 xo[NPC_V];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NPC_V; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    xo[k] = i < nv ? yr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    ss = fmaf(xo[k].x, xo[k].x, fmaf(xo[k].y, xo[k].y, fmaf(xo[k].z, xo[k].z, fmaf(xo[k].w, xo[k].w, ss))));
+  }
+  const float rb = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps_b);
+  ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NPC_V; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    if (i >= nv) continue;
+    const float4 s = sr[i], g = reinterpret_cast<const float4*>(wb)[i];
+    xo[k] = make_float4(s.x + xo[k].x * rb * g.x, s.y + xo[k].y * rb * g.y, s.z + xo[k].z * rb * g.z, s.w + xo[k].w * rb * g.w);
+    sr[i] = xo[k];
+    ss = fmaf(xo[k].x, xo[k].x, fmaf(xo[k].y, xo[k].y, fmaf(xo[k].z, xo[k].z, fmaf(xo[k].w, xo[k].w, ss))));
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  float4* tl = reinterpret_cast<float4*>(tail + (size_t)slots[t] * (K > 1 ? K - 1 : 1) * width);
+#pragma unroll
+  for (int k = 0; k < NPC_V; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    if (i >= nv) continue;
+    const float4 g = reinterpret_cast<const float4*>(w1)[i];
+    float tp[4 * K];                                  // taps of channels 4 i .. 4 i + 3, K each
+#pragma unroll
+    for (int q = 0; q < K; ++q) {
+      const float4 v = reinterpret_cast<const float4*>(taps + (size_t)i * 4 * K)[q];
+      tp[4 * q] = v.x, tp[4 * q + 1] = v.y, tp[4 * q + 2] = v.z, tp[4 * q + 3] = v.w;
+    }
+    const float h0[4] = {xo[k].x * rstd * g.x, xo[k].y * rstd * g.y, xo[k].z * rstd * g.z, xo[k].w * rstd * g.w};
+    float acc[4] = {h0[0], h0[1], h0[2], h0[3]};
+    float4 old[K > 1 ? K - 1 : 1];
+#pragma unroll
+    for (int b = 0; b < K; ++b) {
+      float h[4];
+      if (b == 0) {
+        h[0] = h0[0], h[1] = h0[1], h[2] = h0[2], h[3] = h0[3];
+      } else {
+        const float4 v = tl[(size_t)(K - 1 - b) * nv + i];
+        old[K - 1 - b] = v;
+        h[0] = v.x, h[1] = v.y, h[2] = v.z, h[3] = v.w;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] = fmaf(tp[e * K + (K - 1 - b)], h[e], acc[e]);
+    }
+    store4(xm + (size_t)t * width + 4 * i, acc[0], acc[1], acc[2], acc[3]);
+    if (K > 1) {
+#pragma unroll
+      for (int b = 0; b + 2 < K; ++b) tl[(size_t)b * nv + i] = old[b + 1];
+      tl[(size_t)(K - 2) * nv + i] = make_float4(h0[0], h0[1], h0[2], h0[3]);
+    }
+  }
+}
+
+// y, stream [tokens, width] float32 (every token a row of its own, in slots[token]); wb, w1 [width] and taps [width, K]
+// float32; tail [slots, max(1, K - 1), width] float32; xm [tokens, width] of out_dtype.  Width a multiple of 4 up to
+// 8192, operands 16-byte aligned.
+MIE_EXPORT int mie_branch_norm_conv_single(const float* y, float* stream, const float* wb, float eps_b, const float* w1,
+                                           const float* taps, float* tail, const int* slots, void* xm, int out_dtype, int tokens,
+                                           int width, int K, float eps, hipStream_t s) {
+  if (tokens <= 0) return 0;
+  if (K < 1 || K > CONV_MAX_TAPS) MIE_FAIL("branch_norm_conv_single: %d taps (1 to %d)", K, CONV_MAX_TAPS);
+  if (!y || !stream || !wb || !w1 || !taps || !tail || !slots || !xm) MIE_FAIL("branch_norm_conv_single: a missing operand");
+  if (out_dtype != MIE_F32 && out_dtype != MIE_BF16) MIE_FAIL("branch_norm_conv_single: out dtype code %d", out_dtype);
+  const bool aligned = !(((uintptr_t)y | (uintptr_t)stream | (uintptr_t)wb | (uintptr_t)w1 | (uintptr_t)taps | (uintptr_t)tail |
+                          (uintptr_t)xm) & 15);
+  if (width <= 0 || width % 4 || width > 4 * NPC_V * NORM_THREADS || !aligned)
+    MIE_FAIL("branch_norm_conv_single: width %d (a multiple of 4 up to %d) or an operand that is not 16-byte aligned", width,
+             4 * NPC_V * NORM_THREADS);
+#define BNC_LAUNCH(TO_, K_)                                                                                                   \
+  hipLaunchKernelGGL((branch_norm_conv_single_kernel<TO_, K_>), dim3(tokens), dim3(NORM_THREADS), 0, s, y, stream, wb, eps_b, w1, \
+                     taps, tail, slots, (TO_*)xm, width, eps)
+#define BNC_TAPS(TO_)                                                                                           \
+  switch (K) {                                                                                                  \
+    case 1: BNC_LAUNCH(TO_, 1); break; case 2: BNC_LAUNCH(TO_, 2); break; case 3: BNC_LAUNCH(TO_, 3); break;     \
+    case 4: BNC_LAUNCH(TO_, 4); break; case 5: BNC_LAUNCH(TO_, 5); break; case 6: BNC_LAUNCH(TO_, 6); break;     \
+    case 7: BNC_LAUNCH(TO_, 7); break; default: BNC_LAUNCH(TO_, 8); break;                                       \
+  }
+  if (out_dtype == MIE_F32) { BNC_TAPS(float) } else { BNC_TAPS(bf16) }
+#undef BNC_TAPS
+#undef BNC_LAUNCH
+  MIE_CHECK_LAUNCH("branch_norm_conv_single");
+  return 0;
+}
+
 // ---- t *= factor
 __global__ void scale_kernel(float* __restrict__ t, size_t n, float factor) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) t[i] *= factor;

@@ -52,6 +52,21 @@ class Normed:
         return self._value
 
 
+class NormedBranch:
+    """A branch output that is still to be normed and added to the stream: stream += rmsnorm(y) * weight.  The block
+    that made it hands it on so that the next reader of the stream may do the add in the kernel that makes its own
+    input (``KernelBackend.branch_norm_conv``); anyone else calls ``resolve()``, which performs the add exactly once."""
+
+    def __init__(self, ops, y, stream, weight, eps):
+        self.ops, self.y, self.stream, self.weight, self.eps = ops, y, stream, weight, eps
+
+    def resolve(self):
+        if self.y is not None:
+            self.ops.branch_norm_add(self.y, self.stream, self.weight, self.eps, copy=False)
+            self.y = None
+        return None
+
+
 class StreamCopy:
     """The residual stream as it stands, in the activation dtype (``value``; the stream itself where that is
     float32): what a block hands on when nothing is pending and its branches read the stream unnormed."""
@@ -205,6 +220,13 @@ class KernelBackend:
         h = self.add_rmsnorm(None, stream, w_first, eps, out_dtype=torch.float32)
         x = self.residual_conv(h, taps, tail, step)
         return x, (None if w_second is None else self.add_rmsnorm(None, stream, w_second, eps))
+
+    def branch_norm_conv(self, y, stream, w_out, eps_out, w_next, eps_next, taps, tail, step):
+        """``branch_norm_add`` of y (float32 [T, width]; weight w_out, eps_out) into the float32 stream, then the first
+        result of ``norm_pair_conv`` of the updated stream (weight w_next, eps_next; no second norm) -> x in the
+        activation dtype.  A backend may do both in one kernel."""
+        self.branch_norm_add(y, stream, w_out, eps_out, copy=False)
+        return self.norm_pair_conv(stream, w_next, None, eps_next, taps, tail, step)[0]
 
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
                    layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None,

@@ -800,6 +800,29 @@ class HipBackend(KernelBackend):
                                                   self._stream()))
         return x, y
 
+    def branch_norm_conv(self, y, stream, w_out, eps_out, w_next, eps_next, taps, tail, step):
+        K = taps.shape[1] if taps.dim() == 2 else 0
+        T, W = stream.shape
+        f32 = lambda t: t.dtype == torch.float32 and t.is_contiguous() and t.data_ptr() % 16 == 0      # noqa: E731
+        # steps whose rows are single tokens: one kernel adds the branch and makes the next input
+        if (step.num_rows != T or not 1 <= K <= self.NORM_CONV_MAX_TAPS or W % 4 or W > 8192
+                or not all(f32(t) for t in (y, stream, w_out, w_next, taps, tail))):
+            return super().branch_norm_conv(y, stream, w_out, eps_out, w_next, eps_next, taps, tail, step)
+        self._on_device(y, stream, w_out, w_next, taps, tail)
+        if tuple(y.shape) != (T, W) or tuple(taps.shape) != (W, K) or tuple(tail.shape[1:]) != (max(1, K - 1), W):
+            raise ValueError(f"branch_norm_conv: y {tuple(y.shape)}, taps {tuple(taps.shape)}, tail {tuple(tail.shape)} "
+                             f"for a stream of {(T, W)}")
+        self._f32_vector(w_out, W, "branch_norm_conv: the branch's norm weight")
+        self._f32_vector(w_next, W, "branch_norm_conv: the next norm's weight")
+        if int(step.host["state_slots"].max()) >= tail.shape[0]:
+            raise ValueError("branch_norm_conv: a state slot beyond the tail's slots")
+        x = torch.empty((T, W), dtype=self.act_dtype, device=stream.device)
+        lib = self.lib("embed_norm")
+        library.check(lib, lib.mie_branch_norm_conv_single(_ptr(y), _ptr(stream), _ptr(w_out), float(eps_out), _ptr(w_next),
+                                                           _ptr(taps), _ptr(tail), _ptr(step.state_slots), _ptr(x),
+                                                           _code(self.act_dtype), T, W, K, float(eps_next), self._stream()))
+        return x
+
     LAYOUTS = {"interleaved": 0, "half": 1}
     DELTA_CHUNK = 64         # tokens a chunk of the delta rule's scan; rows up to this long run whole
     DELTA_CHUNKED_MAX_DIM = 128   # wider heads always run whole (the fold keeps a chunk's d x d matrix in the LDS)

@@ -17,6 +17,7 @@ register_kernel_module("embed_norm", {
     "mie_scale": [P, L, F, P],
     "mie_normed_sum_add": [P, P, P, P, P, I, I, F, F, P],
     "mie_norm_pair_conv": [P, P, P, P, P, P, P, P, P, P, I, P, I, I, I, I, F, P],
+    "mie_branch_norm_conv_single": [P, P, P, F, P, P, P, P, P, I, I, I, I, F, P],
 })
 register_kernel_module("rope_kv", {
     "mie_rotary_kv_store": [P, I, L, P, P, P, I, I, I, I, P, P, P, I, I, P],

@@ -7,7 +7,7 @@ be added: the next block's first norm (or the final norm) adds it
 """
 from __future__ import annotations
 
-from ..kernels.api import Normed, Sink, StreamCopy
+from ..kernels.api import Normed, NormedBranch, Sink, StreamCopy
 from .base import Block, CombinedCache, register_block
 
 
@@ -66,6 +66,8 @@ class BranchNormBlock(Block):
 
     def forward(self, h, residual, step, cache, next_norm=None):
         ops = self.ops
+        if isinstance(h, NormedBranch):
+            h = h.resolve()
         if isinstance(h, StreamCopy) and h.stream is residual:
             x = h.value
         else:
@@ -116,6 +118,8 @@ class ParallelBlock(Block):
     def forward(self, h, residual, step, cache, next_norm=None):
         import torch
         ops = self.ops
+        if isinstance(h, NormedBranch):
+            h = h.resolve()
         if isinstance(h, Normed):               # a block of another kind before this one: its last add may be pending
             h = h.pending
         elif isinstance(h, StreamCopy):
@@ -150,7 +154,9 @@ class SandwichBlock(Block):
     norm_feed_forward(stream)))).  ``conv_mixer`` / ``conv_feed_forward`` (c1, c2: parts.ResidualConv or None) keep
     their last inputs beside the mixer's cache (CombinedCache members ``mixer``, ``conv1``, ``conv2``).  The
     feed-forward (with its two norms and its convolution) may be None.  Norms, convolutions and adds are 32-bit;
-    the sublayers hand their 32-bit sums to the norm after them."""
+    the sublayers hand their 32-bit sums to the norm after them.  A sublayer's output is added by whoever reads the
+    stream next (kernels.api.NormedBranch): where that is a sublayer with a convolution, one backend call adds the
+    normed output and makes the next input."""
 
     def __init__(self, norm_mixer, mixer, norm_mixer_out, norm_feed_forward=None, feed_forward=None,
                  norm_feed_forward_out=None, conv_mixer=None, conv_feed_forward=None):
@@ -174,29 +180,41 @@ class SandwichBlock(Block):
                               ("conv1", None if self.conv_mixer is None else self.conv_mixer.cache_requirement()),
                               ("conv2", None if self.conv_feed_forward is None else self.conv_feed_forward.cache_requirement())])
 
-    def _read(self, residual, norm, conv, cache, member, step):
-        """What a sublayer reads: the normed stream, through its convolution if it has one."""
+    def _read(self, pending, residual, norm, conv, cache, member, step):
+        """What a sublayer reads: the normed stream (after the pending branch output, if any, has been added),
+        through its convolution if it has one."""
         import torch
         ops = self.ops
         if conv is None:
+            if pending is not None:
+                pending.resolve()
             return ops.add_rmsnorm(None, residual, norm.weight, norm.eps)
         w = norm.weight if norm.weight.dtype == torch.float32 else norm.weight.float()
-        return ops.norm_pair_conv(residual, w, None, norm.eps, conv.weight, cache.sub(member).tensors["tail"], step)[0]
+        tail = cache.sub(member).tensors["tail"]
+        if pending is not None and pending.y is not None and pending.stream is residual:
+            y, pending.y = pending.y, None
+            return ops.branch_norm_conv(y, residual, pending.weight, pending.eps, w, norm.eps, conv.weight, tail, step)
+        if pending is not None:
+            pending.resolve()
+        return ops.norm_pair_conv(residual, w, None, norm.eps, conv.weight, tail, step)[0]
 
     def forward(self, h, residual, step, cache, next_norm=None):
         ops = self.ops
-        if isinstance(h, Normed):               # a block of another kind before this one: its last add may be pending
+        pending = None
+        if isinstance(h, NormedBranch):         # a block of this kind before this one: its last branch is still to be added
+            pending, h = h, None
+        elif isinstance(h, Normed):             # a block of another kind before this one: its last add may be pending
             h = h.pending
         elif isinstance(h, StreamCopy):
             h = None
         if h is not None:
             residual.add_(h.float())
         combined = self.conv_mixer is not None or self.conv_feed_forward is not None
-        x = self._read(residual, self.norm_mixer, self.conv_mixer, cache, "conv1", step)
+        x = self._read(pending, residual, self.norm_mixer, self.conv_mixer, cache, "conv1", step)
         a = self.mixer.forward(x, step, cache.sub("mixer") if combined else cache)
-        ops.branch_norm_add(a, residual, self.norm_mixer_out.weight, self.norm_mixer_out.eps, copy=False)
+        pending = NormedBranch(ops, a, residual, self.norm_mixer_out.weight, self.norm_mixer_out.eps)
         if self.feed_forward is not None:
-            y = self._read(residual, self.norm_feed_forward, self.conv_feed_forward, cache, "conv2", step)
+            y = self._read(pending, residual, self.norm_feed_forward, self.conv_feed_forward, cache, "conv2", step)
             f = self.feed_forward.forward(y, step)
-            ops.branch_norm_add(f, residual, self.norm_feed_forward_out.weight, self.norm_feed_forward_out.eps, copy=False)
-        return None, residual
+            pending = NormedBranch(ops, f, residual, self.norm_feed_forward_out.weight, self.norm_feed_forward_out.eps)
+        return pending, residual

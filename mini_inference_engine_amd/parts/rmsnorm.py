@@ -8,7 +8,7 @@ the weights are loaded).  The stream and every intermediate are 32-bit; y is rou
 """
 from __future__ import annotations
 
-from ..kernels.api import Normed, StreamCopy
+from ..kernels.api import Normed, NormedBranch, StreamCopy
 from .base import Norm, ParamSpec, register_norm
 
 
@@ -31,6 +31,8 @@ class RMSNorm(Norm):
             self.weight = (1.0 + self.weight.float()).contiguous()
 
     def lazy(self, x, residual, rows=None):
+        if isinstance(x, NormedBranch):     # the block before left a normed branch output to be added: it is added now
+            x = x.resolve()
         if isinstance(x, Normed):
             # the product before this norm already added its result to the stream (and may have prepared
             # this very norm's input)
@@ -42,6 +44,6 @@ class RMSNorm(Norm):
         return Normed(self.ops, x, residual, self.weight, self.eps, rows)
 
     def forward(self, x, residual, rows=None, out_dtype=None):
-        if isinstance(x, (Normed, StreamCopy)):
+        if isinstance(x, (Normed, NormedBranch, StreamCopy)):
             return self.lazy(x, residual, rows).materialize(out_dtype)
         return self.ops.add_rmsnorm(x, residual, self.weight, self.eps, out_dtype=out_dtype, rows=rows)

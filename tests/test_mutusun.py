@@ -707,6 +707,41 @@ def test_activation_on_sums_and_sandwich_norm_kernels(hip, dtype):
         close(stream, want, 2e-6, "stream after a normed branch")
 
 
+class FakeStep:
+    def __init__(self, lens, slots):
+        import numpy as np
+        rs = np.concatenate([[0], np.cumsum(lens)]).astype("int64")
+        self.num_rows, self.num_tokens = len(lens), int(rs[-1])
+        self.host = {"row_start": rs, "state_slots": np.asarray(slots)}
+        self.row_start = torch.tensor(rs, dtype=torch.int32).cuda()
+        self.state_slots = torch.tensor(slots, dtype=torch.int32).cuda()
+        self.token_row = torch.repeat_interleave(torch.arange(len(lens)), torch.tensor(lens)).to(torch.int32).cuda()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_branch_added_and_next_input_made_in_one_kernel(hip, dtype):
+    """Steps of single-token rows add a normed branch output and make the next sublayer's convolved input in one
+    kernel; steps with longer rows in two.  Both against the torch operations, stream, input and tails."""
+    ops, g = hip[dtype], torch.Generator().manual_seed(16)
+    for (W, K, lens, slots) in ((64, 4, [1, 1, 1], [3, 1, 2]), (72, 1, [1], [1]), (2048, 3, [1] * 8, [8, 7, 6, 5, 4, 3, 2, 1]),
+                                (64, 2, [1, 5, 1], [1, 2, 3]), (70, 3, [1, 1], [2, 1])):
+        step = FakeStep(lens, slots)
+        T = step.num_tokens
+        stream, y = _rand((T, W), torch.float32, g), _rand((T, W), torch.float32, g, 3.0)
+        w_out, w_next = _rand((W,), torch.float32, g, 0.4) + 1, _rand((W,), torch.float32, g, 0.4) + 1
+        taps, tail = _rand((W, K), torch.float32, g, 0.5), _rand((9, max(1, K - 1), W), torch.float32, g)
+        want_stream, want_tail = stream.clone(), tail.cpu().clone()
+        ref.ref_branch_norm_add(y, want_stream, w_out, 1e-5, torch.float32)
+        h = ref.ref_add_rmsnorm(None, want_stream.clone(), w_next, 1e-6, torch.float32)
+        want = ref.ref_residual_conv(h.cpu(), taps.cpu(), want_tail, step.host["row_start"], step.host["state_slots"], dtype)
+        got = ops.branch_norm_conv(y, stream, w_out, 1e-5, w_next, 1e-6, taps, tail, step)
+        close(stream, want_stream, 2e-6, f"stream, width {W}, rows {lens}")
+        close(got, want, TOL[dtype] if dtype == torch.bfloat16 else 1e-5, f"input, width {W}, rows {lens}")
+        if K > 1:
+            close(tail, want_tail, 1e-5, f"tails, width {W}, rows {lens}")
+
+
 # ------------------------------------------------------------------------------------------ GPU: whole models
 @pytest.mark.gpu
 def test_keys_just_inside_and_outside_a_chunk_gpu():
