@@ -474,25 +474,27 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, long ld, con
   }
 }
 
-// The same with a token's values kept in the LDS (up to ROUTE_LDS_E router outputs): every logit is read once and
-// every exponential taken once; a chosen output is struck out where it stands.  Same sums in the same order, same
-// choices.
+// The same with a token's values kept in the LDS (up to ROUTE_LDS_E router outputs): the workgroup's 64 tokens' logits
+// come in together, neighbouring threads reading neighbouring numbers (a thread that walked its own row would wait for
+// memory once an output), every exponential is taken once, and a chosen output is struck out where it stands.  Same
+// sums in the same order, same choices.
 #define ROUTE_LDS_E 128
 __global__ void __launch_bounds__(64)
 route_topk_lds_kernel(const float* __restrict__ logits, long ld, const float* __restrict__ bias,
                       const float* __restrict__ choice_bias, int over_all, int* __restrict__ experts,
                       float* __restrict__ shares, int T, int E, int top) {
   __shared__ float sc[ROUTE_LDS_E * 64];
-  const int t = blockIdx.x * 64 + threadIdx.x;
+  const int t0 = blockIdx.x * 64, t = t0 + threadIdx.x;
+  const int here = T - t0 < 64 ? T - t0 : 64;
+  for (int i = threadIdx.x; i < here * E; i += 64) {
+    const int tok = i / E, e = i - tok * E;
+    sc[64 * e + tok] = logits[(size_t)(t0 + tok) * ld + e] + (bias ? bias[e] : 0.f);
+  }
+  __syncthreads();
   if (t >= T) return;
   float* mine = sc + threadIdx.x;            // value e at mine[64 e]: a bank a thread
-  const float* z = logits + (size_t)t * ld;
   float largest = -INFINITY;
-  for (int e = 0; e < E; ++e) {
-    const float v = z[e] + (bias ? bias[e] : 0.f);
-    mine[64 * e] = v;
-    largest = fmaxf(largest, v);
-  }
+  for (int e = 0; e < E; ++e) largest = fmaxf(largest, mine[64 * e]);
   if (over_all) {
     float total = 0.f;
     for (int e = 0; e < E; ++e) total += expf(mine[64 * e] - largest);
