@@ -474,54 +474,53 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, long ld, con
   }
 }
 
-// The same with a token's values kept in the LDS (up to ROUTE_LDS_E router outputs): the workgroup's 64 tokens' logits
-// come in together, neighbouring threads reading neighbouring numbers (a thread that walked its own row would wait for
-// memory once an output), every exponential is taken once, and a chosen output is struck out where it stands.  Same
-// sums in the same order, same choices.
-#define ROUTE_LDS_E 128
-__global__ void __launch_bounds__(64)
-route_topk_lds_kernel(const float* __restrict__ logits, long ld, const float* __restrict__ bias,
-                      const float* __restrict__ choice_bias, int over_all, int* __restrict__ experts,
-                      float* __restrict__ shares, int T, int E, int top) {
-  __shared__ float sc[ROUTE_LDS_E * 64];
-  const int t0 = blockIdx.x * 64, t = t0 + threadIdx.x;
-  const int here = T - t0 < 64 ? T - t0 : 64;
-  for (int i = threadIdx.x; i < here * E; i += 64) {
-    const int tok = i / E, e = i - tok * E;
-    sc[64 * e + tok] = logits[(size_t)(t0 + tok) * ld + e] + (bias ? bias[e] : 0.f);
+// The same with a wave a token (up to ROUTE_WAVE_E router outputs, two a lane): maximum, sum and every choice are
+// reductions over the wave instead of loops of one thread (which wait for each value in turn: 12 us at 18 outputs).
+// A chosen output is struck out in its lane.  The order of a token's sums depends on E alone.
+#define ROUTE_WAVE_E 128
+__global__ void __launch_bounds__(256)
+route_topk_wave_kernel(const float* __restrict__ logits, long ld, const float* __restrict__ bias,
+                       const float* __restrict__ choice_bias, int over_all, int* __restrict__ experts,
+                       float* __restrict__ shares, int T, int E, int top) {
+  const int lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;                        // the whole wave
+  const float* z = logits + (size_t)t * ld;
+  float v[2], c[2];                          // values and choice biases of outputs lane and lane + 64
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < E ? z[e] + (bias ? bias[e] : 0.f) : -INFINITY;
+    c[i] = e < E && over_all && choice_bias ? choice_bias[e] : 0.f;
   }
-  __syncthreads();
-  if (t >= T) return;
-  float* mine = sc + threadIdx.x;            // value e at mine[64 e]: a bank a thread
-  float largest = -INFINITY;
-  for (int e = 0; e < E; ++e) largest = fmaxf(largest, mine[64 * e]);
   if (over_all) {
-    float total = 0.f;
-    for (int e = 0; e < E; ++e) total += expf(mine[64 * e] - largest);
-    for (int e = 0; e < E; ++e) mine[64 * e] = expf(mine[64 * e] - largest) / total;
+    const float largest = wave_max(fmaxf(v[0], v[1]));
+    const float x0 = lane < E ? expf(v[0] - largest) : 0.f, x1 = lane + 64 < E ? expf(v[1] - largest) : 0.f;
+    const float total = wave_sum(x0 + x1);
+    v[0] = lane < E ? x0 / total : -INFINITY;
+    v[1] = lane + 64 < E ? x1 / total : -INFINITY;
   }
-  int* ex = experts + (size_t)t * top;
-  float* sh = shares + (size_t)t * top;
+  float mine = 0.f;                          // lane j keeps the value of choice j
   for (int j = 0; j < top; ++j) {
-    int best = -1;
-    float bv = 0.f, bs = 0.f;
-    for (int e = 0; e < E; ++e) {
-      const float s = mine[64 * e];
-      if (s == -INFINITY) continue;            // struck out
-      const float v = over_all && choice_bias ? s + choice_bias[e] : s;
-      if (best < 0 || v > bv) { best = e; bv = v; bs = s; }
+    const float k0 = v[0] + c[0], k1 = v[1] + c[1];          // a struck or missing output stays -inf
+    const float m = wave_max(fmaxf(k0, k1));
+    int best = k0 == m ? lane : (k1 == m ? lane + 64 : 1 << 30);   // lowest index first among equals
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const int other = __shfl_xor(best, o, MIE_WAVE);
+      best = other < best ? other : best;
     }
-    if (best < 0) best = 0;                    // every value left is -inf: cannot happen with finite logits
-    ex[j] = best;
-    sh[j] = bs;
-    mine[64 * best] = -INFINITY;
+    if (best >= E) best = 0;                 // every value left is -inf or a NaN: cannot happen with finite logits
+    const float s = __shfl(best < 64 ? v[0] : v[1], best & 63, MIE_WAVE);
+    if (lane == (best & 63)) v[best >> 6] = -INFINITY;
+    if (lane == j) mine = s;
+    if (lane == 0) experts[(size_t)t * top + j] = best;
   }
   if (!over_all) {
-    float sum = 0.f;
-    const float first = sh[0];
-    for (int j = 0; j < top; ++j) sum += expf(sh[j] - first);
-    for (int j = 0; j < top; ++j) sh[j] = expf(sh[j] - first) / sum;
+    const float first = __shfl(mine, 0, MIE_WAVE);
+    mine = lane < top ? expf(mine - first) : 0.f;
+    mine /= wave_sum(mine);
   }
+  if (lane < top) shares[(size_t)t * top + lane] = mine;
 }
 
 static int route_topk_launch(const float* logits, long ld, const float* bias, const float* choice_bias, int over_all,
@@ -529,8 +528,8 @@ static int route_topk_launch(const float* logits, long ld, const float* bias, co
   if (T <= 0) return 0;
   if (E <= 0 || top <= 0 || top > E || top > ROUTE_MAX_TOP) MIE_FAIL("route_topk: top %d of %d experts (at most %d)", top, E, ROUTE_MAX_TOP);
   if (ld < E) MIE_FAIL("route_topk: row stride %ld < %d", ld, E);
-  if (E <= ROUTE_LDS_E)
-    hipLaunchKernelGGL(route_topk_lds_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, ld, bias, choice_bias, over_all,
+  if (E <= ROUTE_WAVE_E)
+    hipLaunchKernelGGL(route_topk_wave_kernel, dim3((T + 3) / 4), dim3(256), 0, s, logits, ld, bias, choice_bias, over_all,
                        experts, shares, T, E, top);
   else
     hipLaunchKernelGGL(route_topk_kernel, dim3((T + 63) / 64), dim3(64), 0, s, logits, ld, bias, choice_bias, over_all, experts,

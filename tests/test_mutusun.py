@@ -77,7 +77,17 @@ C1 = att(3, 1, 10, vdim=14, scale=0.4, softcap=9.0, chunk=5)
 CFG_C = model(101, 70, 1e-6, 1, [layer(C1, moe(3, 1, 2, 26, 2.5)),
                                  layer(C1, dict(kind="dense", ff=50)),
                                  layer(att(5, 5, 6, chunk=33), moe(2, 2, 2, 18, 0.5))])
-CONFIGS = {"A": (CFG_A, 3), "B": (CFG_B, 4), "C": (CFG_C, 6)}
+# a routed layer first, eight query heads on one key head, values wider than keys, a chunk longer than most requests,
+# five taps, more router outputs than a token's choices by far
+D1 = att(8, 1, 40, vdim=56, scale=0.2, softcap=12.0, chunk=100)          # heads padded to 64
+D2 = att(2, 2, 72, softcap=3.0, chunk=50)                                # heads padded to 80
+M4 = moe(9, 3, 6, 32, 4.0)
+CFG_D = model(333, 96, 1e-4, 5, [layer(D1, M4),
+                                 layer(D2, dict(kind="dense", ff=200)),
+                                 layer(D1, M4, weights_of=0),
+                                 layer(D2, dict(kind="dense", ff=200), weights_of=1),
+                                 layer(D1, None)])
+CONFIGS = {"A": (CFG_A, 3), "B": (CFG_B, 4), "C": (CFG_C, 6), "D": (CFG_D, 8)}
 
 
 def shape_weights(cfg, seed, sharp=True):
