@@ -12,7 +12,8 @@
 // step holds and however the request was cut into steps.  With a sink, one more term exp(sink)
 // joins the softmax's denominator at the end and has no value.  With a cap c the scaled scores
 // pass through c * tanh(score / c).  In the sigmoid mode there is no softmax: a visible key counts
-// with sigmoid(score + the head's bias), and the weights are not normalised.
+// with sigmoid(score + the head's bias), and the weights are not normalised.  With a distance bias a key n
+// positions back adds a number of its head's table to the score.
 //
 // This is the reference kernel of the engine: the float32 path runs on it, and the
 // bfloat16 path uses it wherever a faster kernel does not take the shape.
@@ -45,7 +46,8 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
                        const T* __restrict__ v_cache, T* __restrict__ out, const int* __restrict__ block_tables,
                        int max_blocks, const int* __restrict__ token_row, const int* __restrict__ positions, int Hq,
                        int Hkv, int D, int page, float scale, int window, int has_sink, float sink, int chunk,
-                       float softcap, int sigmoid, const float* __restrict__ head_bias) {
+                       float softcap, int sigmoid, const float* __restrict__ head_bias,
+                       const float* __restrict__ dist_bias, int dist_n) {
   __shared__ float qs[NR * 64];
   __shared__ float ps[64];
   __shared__ long long base[64];     // per key of the chunk: offset of its value column
@@ -55,6 +57,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
   int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
   if (chunk > 0 && pos / chunk * chunk > lo) lo = pos / chunk * chunk;
   const float hb = sigmoid && head_bias ? head_bias[h] : 0.f;
+  const float* db = dist_bias ? dist_bias + (size_t)h * dist_n : nullptr;
   const int* bt = block_tables + (size_t)row * max_blocks;
   const T* qp = q + (size_t)t * q_stride + (size_t)h * D;
   for (int d = lane; d < D; d += 64) qs[d] = to_float(qp[d]);
@@ -84,6 +87,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
       }
       s = dot * scale;
       if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      if (db) s += db[pos - key < dist_n ? pos - key : dist_n - 1];
     }
     float alpha = 1.f, p;
     if (sigmoid) {
@@ -133,8 +137,9 @@ static int paged_attention_launch(const void* q, long q_stride, const void* k_ca
                                    int dtype, const int* block_tables, int max_blocks, const int* token_row,
                                    const int* positions, int tokens, int Hq, int Hkv, int D, int page, float scale,
                                    int window, int has_sink, float sink, int chunk, float softcap, int sigmoid,
-                                   const float* head_bias, hipStream_t stream) {
+                                   const float* head_bias, const float* dist_bias, int dist_n, hipStream_t stream) {
   if (tokens <= 0) return 0;
+  if (dist_bias && dist_n < 1) MIE_FAIL("paged_attention: a distance bias of %d entries a head", dist_n);
   if (chunk < 0 || softcap < 0.f) MIE_FAIL("paged_attention: chunk %d, score cap %g", chunk, (double)softcap);
   if (sigmoid && has_sink) MIE_FAIL("paged_attention: a sink belongs to a softmax; the weights asked for are sigmoids");
   if (D % 16 || D < 16 || D > ATT_MAX_D) MIE_FAIL("paged_attention: head_dim %d (multiples of 16 up to %d)", D, ATT_MAX_D);
@@ -146,7 +151,7 @@ static int paged_attention_launch(const void* q, long q_stride, const void* k_ca
 #define PA_LAUNCH(T_, NR_)                                                                                               \
   hipLaunchKernelGGL((paged_attention_kernel<T_, NR_>), grid, block, 0, stream, (const T_*)q, q_stride, (const T_*)k_cache, \
                      (const T_*)v_cache, (T_*)out, block_tables, max_blocks, token_row, positions, Hq, Hkv, D, page, scale,  \
-                     window, has_sink, sink, chunk, softcap, sigmoid, head_bias)
+                     window, has_sink, sink, chunk, softcap, sigmoid, head_bias, dist_bias, dist_n)
   if (dtype == MIE_F32 && D <= 256) PA_LAUNCH(float, 4);
   else if (dtype == MIE_F32) PA_LAUNCH(float, 16);
   else if (dtype == MIE_BF16 && D <= 256) PA_LAUNCH(bf16, 4);
@@ -162,17 +167,20 @@ MIE_EXPORT int mie_paged_attention(const void* q, long q_stride, const void* k_c
                                    const int* positions, int tokens, int Hq, int Hkv, int D, int page, float scale,
                                    int window, int has_sink, float sink, hipStream_t stream) {
   return paged_attention_launch(q, q_stride, k_cache, v_cache, out, dtype, block_tables, max_blocks, token_row, positions,
-                                tokens, Hq, Hkv, D, page, scale, window, has_sink, sink, 0, 0.f, 0, nullptr, stream);
+                                tokens, Hq, Hkv, D, page, scale, window, has_sink, sink, 0, 0.f, 0, nullptr, nullptr, 0, stream);
 }
 
 // The same with what a design may put between scores and weights: a chunk size (0: none), a cap on the scores
-// (0: none), sigmoid weights with a bias per query head (head_bias float32 [Hq] or null) instead of the softmax.
+// (0: none), sigmoid weights with a bias per query head (head_bias float32 [Hq] or null) instead of the softmax, a bias
+// on the score by the key's distance (dist_bias float32 [Hq, dist_n] or null: a key n positions back adds entry
+// min(n, dist_n - 1) of the head's row, after scale and cap).
 MIE_EXPORT int mie_paged_attention_scored(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
                                           int dtype, const int* block_tables, int max_blocks, const int* token_row,
                                           const int* positions, int tokens, int Hq, int Hkv, int D, int page, float scale,
                                           int window, int has_sink, float sink, int chunk, float softcap, int sigmoid,
-                                          const float* head_bias, hipStream_t stream) {
+                                          const float* head_bias, const float* dist_bias, int dist_n,
+                                          hipStream_t stream) {
   return paged_attention_launch(q, q_stride, k_cache, v_cache, out, dtype, block_tables, max_blocks, token_row, positions,
                                 tokens, Hq, Hkv, D, page, scale, window, has_sink, sink, chunk, softcap, sigmoid, head_bias,
-                                stream);
+                                dist_bias, dist_n, stream);
 }

@@ -225,7 +225,7 @@ MIE_EXPORT int mie_act_mul(const void* gu, long ld_in, void* out, long ld_out, i
 // ---- elementwise steps on a product's float32 sums, rounded once on the way out
 // act_store: out[r, i] = act(in[r, i]).  clamped_glu: in holds gate sums [0, inner) and up sums [inner, 2 inner) of a
 // row (block 0), or alternating blocks of ``block`` gate sums and ``block`` up sums (inner a multiple of block);
-// out[r, i] = g * sigmoid(alpha g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit).
+// out[r, i] = g * sigmoid(alpha g) * (u + shift) with g = min(gate, limit), u = clamp(up, -limit, limit).
 template <typename TO>
 __global__ void __launch_bounds__(256)
 act_store_kernel(const float* __restrict__ in, long ld_in, TO* __restrict__ out, long ld_out, int rows, int n, int act) {
@@ -239,14 +239,14 @@ act_store_kernel(const float* __restrict__ in, long ld_in, TO* __restrict__ out,
 template <typename TO>
 __global__ void __launch_bounds__(256)
 clamped_glu_kernel(const float* __restrict__ in, long ld_in, TO* __restrict__ out, long ld_out, int rows, int inner,
-                   float limit, float alpha, int block) {
+                   float limit, float alpha, float shift, int block) {
   const size_t total = (size_t)rows * inner;
   for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
     const size_t r = e / inner, i = e - r * inner;
     const size_t gi = block ? i / block * 2 * block + i % block : i, ui = block ? gi + block : inner + i;
     const float g = fminf(in[r * ld_in + gi], limit);
     const float u = fminf(fmaxf(in[r * ld_in + ui], -limit), limit);
-    out[r * ld_out + i] = from_float<TO>(g * mie_sigmoid(alpha * g) * (u + 1.0f));
+    out[r * ld_out + i] = from_float<TO>(g * mie_sigmoid(alpha * g) * (u + shift));
   }
 }
 
@@ -269,7 +269,7 @@ MIE_EXPORT int mie_act_store(const float* in, long ld_in, void* out, long ld_out
 }
 
 MIE_EXPORT int mie_clamped_glu(const float* in, long ld_in, void* out, long ld_out, int out_dtype, int rows, int inner,
-                               float limit, float alpha, int block, hipStream_t s) {
+                               float limit, float alpha, float shift, int block, hipStream_t s) {
   if (rows <= 0 || inner <= 0) return 0;
   if (block < 0 || (block && inner % block)) MIE_FAIL("clamped_glu: blocks of %d in an inner size of %d", block, inner);
   if (ld_in < 2L * inner || ld_out < inner) MIE_FAIL("clamped_glu: leading dims %ld, %ld for inner size %d", ld_in, ld_out, inner);
@@ -278,9 +278,9 @@ MIE_EXPORT int mie_clamped_glu(const float* in, long ld_in, void* out, long ld_o
   int blocks = (int)((total + 255) / 256);
   if (blocks > 16384) blocks = 16384;
   if (out_dtype == MIE_F32)
-    hipLaunchKernelGGL(clamped_glu_kernel<float>, dim3(blocks), dim3(256), 0, s, in, ld_in, (float*)out, ld_out, rows, inner, limit, alpha, block);
+    hipLaunchKernelGGL(clamped_glu_kernel<float>, dim3(blocks), dim3(256), 0, s, in, ld_in, (float*)out, ld_out, rows, inner, limit, alpha, shift, block);
   else if (out_dtype == MIE_BF16)
-    hipLaunchKernelGGL(clamped_glu_kernel<bf16>, dim3(blocks), dim3(256), 0, s, in, ld_in, (bf16*)out, ld_out, rows, inner, limit, alpha, block);
+    hipLaunchKernelGGL(clamped_glu_kernel<bf16>, dim3(blocks), dim3(256), 0, s, in, ld_in, (bf16*)out, ld_out, rows, inner, limit, alpha, shift, block);
   else
     MIE_FAIL("clamped_glu: dtype code %d", out_dtype);
   MIE_CHECK_LAUNCH("clamped_glu");

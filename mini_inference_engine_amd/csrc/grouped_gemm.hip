@@ -28,8 +28,8 @@ struct GroupedArgs {
   int M, N, K, G, act;
   const void* zeros;            // 64 bytes of zeros in device memory: what a load beyond a tile's rows or beyond K reads
   // glu != 0 (matrix-core kernel only): W's rows alternate in blocks of 16 gate rows and 16 up rows, and C [.., N / 2]
-  // receives g * sigmoid(glu_alpha g) * (u + 1), g = min(gate sum, glu_limit), u = clamp(up sum, -glu_limit, glu_limit)
-  int glu; float glu_limit, glu_alpha;
+  // receives g * sigmoid(glu_alpha g) * (u + glu_shift), g = min(gate sum, glu_limit), u = clamp(up sum, -glu_limit, glu_limit)
+  int glu; float glu_limit, glu_alpha, glu_shift;
 };
 
 template <typename TA, typename TW, typename TC>
@@ -311,7 +311,7 @@ grouped_gemm_ring_kernel(GroupedArgs p) {
           if (m >= m_end) continue;
           const float gt = fminf(acc[i][2 * jj][e], p.glu_limit);
           const float up = fminf(fmaxf(acc[i][2 * jj + 1][e], -p.glu_limit), p.glu_limit);
-          C[(size_t)(c_row0 + m) * p.ldc + n] = from_float<TC>(gt * mie_sigmoid(p.glu_alpha * gt) * (up + 1.0f));
+          C[(size_t)(c_row0 + m) * p.ldc + n] = from_float<TC>(gt * mie_sigmoid(p.glu_alpha * gt) * (up + p.glu_shift));
         }
     }
     return;
@@ -365,7 +365,7 @@ static int grouped_linear_run(const void* A, int a_dtype, long lda, long a_group
                               long ldw, long w_group, void* C, int c_dtype, long ldc, long c_group, const float* bias,
                               const float* gate, long ldg, const int* offs, const int* gather, int gather_div, int M,
                               int N, int K, int G, int act, const void* zeros, int glu, float glu_limit, float glu_alpha,
-                              hipStream_t s) {
+                              float glu_shift, hipStream_t s) {
   if (M <= 0 || N <= 0 || G <= 0) return 0;
   if (K <= 0 || !A || !W || !C) MIE_FAIL("grouped_linear: K %d or a null operand", K);
   if (lda < K && !offs && a_group == 0) MIE_FAIL("grouped_linear: A row stride %ld < K %d", lda, K);
@@ -376,7 +376,7 @@ static int grouped_linear_run(const void* A, int a_dtype, long lda, long a_group
   if (gather && gather_div <= 0) MIE_FAIL("grouped_linear: gather divisor %d", gather_div);
   if (act < MIE_ACT_NONE || act > MIE_ACT_RELU2) MIE_FAIL("grouped_linear: activation code %d", act);
   GroupedArgs p = {A, lda, offs ? 0 : a_group, offs ? 1 : a_mod, W, ldw, w_group, C, ldc, offs ? 0 : c_group, bias, gate, ldg,
-                   offs, gather, gather_div, M, N, K, G, act, zeros, glu, glu_limit, glu_alpha};
+                   offs, gather, gather_div, M, N, K, G, act, zeros, glu, glu_limit, glu_alpha, glu_shift};
   const long mt = (M + GG_T - 1) / GG_T + (offs ? G : 0);
   if (mt > 65535 || G > 65535) MIE_FAIL("grouped_linear: %ld row tiles, %d groups are beyond the grid", mt, G);
   dim3 grid((N + GG_T - 1) / GG_T, (unsigned)mt, offs ? 1 : G);
@@ -411,24 +411,25 @@ MIE_EXPORT int mie_grouped_linear(const void* A, int a_dtype, long lda, long a_g
                                   const float* gate, long ldg, const int* offs, const int* gather, int gather_div, int M,
                                   int N, int K, int G, int act, const void* zeros, hipStream_t s) {
   return grouped_linear_run(A, a_dtype, lda, a_group, a_mod, W, w_dtype, ldw, w_group, C, c_dtype, ldc, c_group, bias, gate, ldg,
-                            offs, gather, gather_div, M, N, K, G, act, zeros, 0, 0.f, 0.f, s);
+                            offs, gather, gather_div, M, N, K, G, act, zeros, 0, 0.f, 0.f, 0.f, s);
 }
 
 // The same in the rows shape for gated experts, on the matrix cores only (bfloat16 A and W, K and the strides multiples
 // of 8): W's N rows alternate in blocks of 16 gate rows and 16 up rows, C [rows, N / 2] receives
-// g * sigmoid(alpha g) * (u + 1) with g = min(gate sum, limit), u = clamp(up sum, -limit, limit).
+// g * sigmoid(alpha g) * (u + shift) with g = min(gate sum, limit), u = clamp(up sum, -limit, limit) (an infinite limit
+// clamps nothing).
 MIE_EXPORT int mie_grouped_glu(const void* A, int a_dtype, long lda, const void* W, int w_dtype, long ldw, long w_group, void* C,
                                int c_dtype, long ldc, const int* offs, const int* gather, int gather_div, int M, int N, int K,
-                               int G, float limit, float alpha, const void* zeros, hipStream_t s) {
+                               int G, float limit, float alpha, float shift, const void* zeros, hipStream_t s) {
   if (!offs || !zeros) MIE_FAIL("grouped_glu: group offsets and the block of zeros are needed");
   return grouped_linear_run(A, a_dtype, lda, 0, 1, W, w_dtype, ldw, w_group, C, c_dtype, ldc, 0, nullptr, nullptr, 0, offs, gather,
-                            gather_div, M, N, K, G, MIE_ACT_NONE, zeros, 1, limit, alpha, s);
+                            gather_div, M, N, K, G, MIE_ACT_NONE, zeros, 1, limit, alpha, shift, s);
 }
 
 // ---- router, one thread a token.  over_all == 0: the `top` largest of logits[t, :] + bias (lowest index first among
 // equals), in falling order, and the softmax over those alone.  over_all != 0: scores = softmax of logits + bias over
 // all E; chosen are the `top` largest of scores + choice_bias (same order rules); the shares are the chosen ones'
-// scores as they are.
+// scores as they are (over_all == 1) or divided by their sum + 1e-20 (over_all == 2).
 #define ROUTE_MAX_TOP 16
 __global__ void route_topk_kernel(const float* __restrict__ logits, long ld, const float* __restrict__ bias,
                                   const float* __restrict__ choice_bias, int over_all, int* __restrict__ experts,
@@ -467,6 +468,10 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, long ld, con
     const float first = val[0];
     for (int j = 0; j < top; ++j) { val[j] = expf(val[j] - first); sum += val[j]; }
     for (int j = 0; j < top; ++j) val[j] /= sum;
+  } else if (over_all == 2) {
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) sum += val[j];
+    for (int j = 0; j < top; ++j) val[j] /= sum + 1e-20f;
   }
   for (int j = 0; j < top; ++j) {
     experts[(size_t)t * top + j] = chosen[j];
@@ -519,6 +524,9 @@ route_topk_wave_kernel(const float* __restrict__ logits, long ld, const float* _
     const float first = __shfl(mine, 0, MIE_WAVE);
     mine = lane < top ? expf(mine - first) : 0.f;
     mine /= wave_sum(mine);
+  } else if (over_all == 2) {
+    mine = lane < top ? mine : 0.f;
+    mine /= wave_sum(mine) + 1e-20f;
   }
   if (lane < top) shares[(size_t)t * top + lane] = mine;
 }
@@ -544,8 +552,8 @@ MIE_EXPORT int mie_route_topk(const float* logits, long ld, const float* bias, i
 }
 
 MIE_EXPORT int mie_route_topk_all(const float* logits, long ld, const float* bias, const float* choice_bias, int* experts,
-                                  float* shares, int T, int E, int top, hipStream_t s) {
-  return route_topk_launch(logits, ld, bias, choice_bias, 1, experts, shares, T, E, top, s);
+                                  float* shares, int T, int E, int top, int renormalise, hipStream_t s) {
+  return route_topk_launch(logits, ld, bias, choice_bias, renormalise ? 2 : 1, experts, shares, T, E, top, s);
 }
 
 // ---- sort the n = T * top (token, choice) pairs by expert: offs [E + 1] (where each expert's pairs start in the

@@ -5,8 +5,8 @@
 //   the value column [c | 0], both padded to P numbers, in the layouts the attention kernels read
 //   (keys [pages, 1, page, P], values [pages, 1, P, page]).
 // latent_query_rotate: the rotated part of every query head ([T, H, P]: columns kv_rank .. kv_rank + rot_dim), turned in place.
-// Rotation: elements 2i and 2i + 1 turn by the angle position * inv_freq[i], for i < n_freq; angle, cosine and sine
-// in 32-bit; elements beyond 2 n_freq pass unchanged.
+// Rotation: elements 2i and 2i + 1 (or, in the half layout, i and i + n_freq) turn by the angle position * inv_freq[i],
+// for i < n_freq; angle, cosine and sine in 32-bit; elements beyond 2 n_freq pass unchanged.
 #include "common.hpp"
 
 __device__ __forceinline__ void turn_pair(float u, float v, int pos, float inv_freq, float& ou, float& ov) {
@@ -21,7 +21,7 @@ latent_kv_store_kernel(const float* __restrict__ sums, long ld, const TW* __rest
                        const int* __restrict__ positions, const float* __restrict__ inv_freq, int n_freq,
                        TC* __restrict__ k_cache, TC* __restrict__ v_cache, const int* __restrict__ slots, int kv_rank,
                        int rot_dim, int P, int page, const float* __restrict__ q_sums, const TW* __restrict__ q_weight,
-                       TC* __restrict__ q_out, int q_rank) {
+                       TC* __restrict__ q_out, int q_rank, int half_layout) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   if (q_out) {                      // the query latent of the same token, normed beside it (one kernel less a layer)
@@ -45,13 +45,14 @@ latent_kv_store_kernel(const float* __restrict__ sums, long ld, const TW* __rest
     vc[(size_t)i * page] = c;
   }
   const float* r = x + kv_rank;
-  for (int i = threadIdx.x; i < rot_dim / 2; i += blockDim.x) {
-    float u = r[2 * i], v = r[2 * i + 1];
-    if (i < n_freq) turn_pair(u, v, pos, inv_freq[i], u, v);
-    kr[kv_rank + 2 * i] = from_float<TC>(u);
-    kr[kv_rank + 2 * i + 1] = from_float<TC>(v);
+  for (int i = threadIdx.x; i < n_freq; i += blockDim.x) {          // the turned pairs
+    const int d1 = half_layout ? i : 2 * i, d2 = half_layout ? i + n_freq : 2 * i + 1;
+    float u, v;
+    turn_pair(r[d1], r[d2], pos, inv_freq[i], u, v);
+    kr[kv_rank + d1] = from_float<TC>(u);
+    kr[kv_rank + d2] = from_float<TC>(v);
   }
-  if ((rot_dim & 1) && threadIdx.x == 0) kr[kv_rank + rot_dim - 1] = from_float<TC>(r[rot_dim - 1]);
+  for (int i = 2 * n_freq + threadIdx.x; i < rot_dim; i += blockDim.x) kr[kv_rank + i] = from_float<TC>(r[i]);
   for (int i = kv_rank + rot_dim + threadIdx.x; i < P; i += blockDim.x) kr[i] = from_float<TC>(0.f);
   for (int i = kv_rank + threadIdx.x; i < P; i += blockDim.x) vc[(size_t)i * page] = from_float<TC>(0.f);
 }
@@ -64,7 +65,8 @@ MIE_EXPORT const char* latent_attention_last_error() { return g_mie_error; }
 MIE_EXPORT int mie_latent_kv_store(const float* sums, long ld, const void* norm_weight, int w_dtype, float eps,
                                    const int* positions, const float* inv_freq, int n_freq, void* k_cache, void* v_cache,
                                    int cache_dtype, const int* slots, int tokens, int kv_rank, int rot_dim, int P, int page,
-                                   const float* q_sums, const void* q_weight, void* q_out, int q_rank, hipStream_t s) {
+                                   const float* q_sums, const void* q_weight, void* q_out, int q_rank, int half_layout,
+                                   hipStream_t s) {
   if (tokens <= 0) return 0;
   if (kv_rank <= 0 || rot_dim < 0 || P < kv_rank + rot_dim || page <= 0 || 2 * n_freq > rot_dim)
     MIE_FAIL("latent_kv_store: kv_rank %d, rot_dim %d, padded %d, page %d, %d turned pairs", kv_rank, rot_dim, P, page, n_freq);
@@ -74,7 +76,7 @@ MIE_EXPORT int mie_latent_kv_store(const float* sums, long ld, const void* norm_
 #define LKV(TW_, TC_)                                                                                                     \
   hipLaunchKernelGGL((latent_kv_store_kernel<TW_, TC_>), dim3(tokens), dim3(256), 0, s, sums, ld, (const TW_*)norm_weight, \
                      eps, positions, inv_freq, n_freq, (TC_*)k_cache, (TC_*)v_cache, slots, kv_rank, rot_dim, P, page, \
-                     q_sums, (const TW_*)q_weight, (TC_*)q_out, q_rank)
+                     q_sums, (const TW_*)q_weight, (TC_*)q_out, q_rank, half_layout)
   if (w_dtype == MIE_F32 && cache_dtype == MIE_F32) LKV(float, float);
   else if (w_dtype == MIE_F32 && cache_dtype == MIE_BF16) LKV(float, bf16);
   else if (w_dtype == MIE_BF16 && cache_dtype == MIE_F32) LKV(bf16, float);
@@ -85,33 +87,36 @@ MIE_EXPORT int mie_latent_kv_store(const float* sums, long ld, const void* norm_
   return 0;
 }
 
-// q [tokens, H, P] (rows ldq apart): the pairs (2i, 2i + 1), i < n_freq, of columns kv_rank .. of every head turn in place.
+// q [tokens, H, P] (rows ldq apart): the pairs (2i, 2i + 1) (half layout: (i, i + n_freq)), i < n_freq, of columns kv_rank .. of
+// every head turn in place.
 template <typename T>
 __global__ void latent_query_rotate_kernel(T* __restrict__ q, long ldq, const int* __restrict__ positions,
-                                           const float* __restrict__ inv_freq, int n_freq, int H, int kv_rank, int P) {
+                                           const float* __restrict__ inv_freq, int n_freq, int H, int kv_rank, int P,
+                                           int half_layout) {
   const int t = blockIdx.x, pos = positions[t];
   for (int idx = threadIdx.x; idx < H * n_freq; idx += blockDim.x) {
     const int h = idx / n_freq, i = idx - h * n_freq;
-    T* pair = q + (size_t)t * ldq + (size_t)h * P + kv_rank + 2 * i;
+    T* part = q + (size_t)t * ldq + (size_t)h * P + kv_rank;
+    const int d1 = half_layout ? i : 2 * i, d2 = half_layout ? i + n_freq : 2 * i + 1;
     float u, v;
-    turn_pair(to_float(pair[0]), to_float(pair[1]), pos, inv_freq[i], u, v);
-    pair[0] = from_float<T>(u);
-    pair[1] = from_float<T>(v);
+    turn_pair(to_float(part[d1]), to_float(part[d2]), pos, inv_freq[i], u, v);
+    part[d1] = from_float<T>(u);
+    part[d2] = from_float<T>(v);
   }
 }
 
 MIE_EXPORT int mie_latent_query_rotate(void* q, long ldq, int dtype, const int* positions, const float* inv_freq, int n_freq,
-                                       int tokens, int H, int kv_rank, int P, hipStream_t s) {
+                                       int tokens, int H, int kv_rank, int P, int half_layout, hipStream_t s) {
   if (tokens <= 0 || n_freq <= 0) return 0;
   if (H <= 0 || kv_rank < 0 || P < kv_rank + 2 * n_freq || ldq < (long)H * P)
     MIE_FAIL("latent_query_rotate: %d heads of %d, latent %d, %d turned pairs, row stride %ld", H, P, kv_rank, n_freq, ldq);
   if (!q || !positions || !inv_freq) MIE_FAIL("latent_query_rotate: operands");
   if (dtype == MIE_F32)
     hipLaunchKernelGGL(latent_query_rotate_kernel<float>, dim3(tokens), dim3(128), 0, s, (float*)q, ldq, positions, inv_freq, n_freq,
-                       H, kv_rank, P);
+                       H, kv_rank, P, half_layout);
   else if (dtype == MIE_BF16)
     hipLaunchKernelGGL(latent_query_rotate_kernel<bf16>, dim3(tokens), dim3(128), 0, s, (bf16*)q, ldq, positions, inv_freq, n_freq,
-                       H, kv_rank, P);
+                       H, kv_rank, P, half_layout);
   else
     MIE_FAIL("latent_query_rotate: dtype code %d", dtype);
   MIE_CHECK_LAUNCH("latent_query_rotate");

@@ -52,19 +52,45 @@ class Normed:
         return self._value
 
 
+class NormedLayer(Normed):
+    """The same for a layer norm with weight and bias: layernorm(residual (+ pending)) * weight + bias."""
+
+    def __init__(self, ops, pending, residual, weight, bias, eps, rows=None):
+        super().__init__(ops, pending, residual, weight, eps, rows)
+        self.bias = bias
+
+    def with_rows(self, rows):
+        return NormedLayer(self.ops, self.pending, self.residual, self.weight, self.bias, self.eps, rows)
+
+    def materialize(self, out_dtype=None):
+        if self._value is None:
+            self._value = self.ops.add_layernorm(self.pending, self.residual, self.weight, self.bias, self.eps,
+                                                 out_dtype=out_dtype, rows=self.rows)
+            if self.rows is None:
+                self.pending = None
+        return self._value
+
+
 class NormedBranch:
-    """A branch output that is still to be normed and added to the stream: stream += rmsnorm(y) * weight.  The block
+    """A branch output that is still to be normed and added to the stream: stream += rmsnorm(y) * weight, or, with
+    ``norm`` (a parts.Norm that has ``add_branch``), stream += norm(y) whatever kind of norm that is.  The block
     that made it hands it on so that the next reader of the stream may do the add in the kernel that makes its own
-    input (``KernelBackend.branch_norm_conv``); anyone else calls ``resolve()``, which performs the add exactly once."""
+    input (``KernelBackend.branch_norm_conv``, or ``resolve(then=...)``); anyone else calls ``resolve()``, which
+    performs the add exactly once."""
 
-    def __init__(self, ops, y, stream, weight, eps):
-        self.ops, self.y, self.stream, self.weight, self.eps = ops, y, stream, weight, eps
+    def __init__(self, ops, y, stream, weight, eps, norm=None):
+        self.ops, self.y, self.stream, self.weight, self.eps, self.norm = ops, y, stream, weight, eps, norm
 
-    def resolve(self):
-        if self.y is not None:
-            self.ops.branch_norm_add(self.y, self.stream, self.weight, self.eps, copy=False)
-            self.y = None
-        return None
+    def resolve(self, then=None):
+        """Adds the normed branch output to the stream.  ``then`` (a parts.Norm): also returns that norm of the updated
+        stream, in the activation dtype; where both norms are of one kind that knows how, in the same kernel."""
+        y, self.y = self.y, None
+        if y is None:
+            return None if then is None else then.forward(None, self.stream)
+        if self.norm is not None:
+            return self.norm.add_branch(y, self.stream, then)
+        self.ops.branch_norm_add(y, self.stream, self.weight, self.eps, copy=False)
+        return None if then is None else then.forward(None, self.stream)
 
 
 class StreamCopy:
@@ -123,6 +149,23 @@ class KernelBackend:
         """t *= factor in place (float32), returns t."""
         raise NotImplementedError
 
+    def scale_softcap_(self, t, scale, cap):
+        """t = cap * tanh(t * scale / cap) in place (float32; ``cap`` None: t * scale), returns t."""
+        raise NotImplementedError
+
+    def add_layernorm(self, x, residual, weight, bias, eps, out_dtype=None, rows=None):
+        """If ``x`` is given: residual += float(x), in place.  y = (residual - mean) / sqrt(var + eps) * weight + bias,
+        mean and var (the mean of the squared deviations) of each row, all in float32 (weight, bias float32 [width]),
+        rounded once to ``out_dtype`` (default act_dtype).  With ``rows`` only those rows are computed, y is
+        [len(rows), width] and residual is not modified."""
+        raise NotImplementedError
+
+    def branch_layernorm_add(self, y, stream, weight, bias, eps, next_norm=None):
+        """stream += layernorm(y) * weight + bias, row by row in float32 (y [T, width] of any float dtype).  With
+        ``next_norm`` = (weight, bias, eps) also returns that layer norm of the updated stream in the activation dtype
+        (a backend may do both in one kernel); else None."""
+        raise NotImplementedError
+
     def branch_norm_add(self, y, stream, weight, eps, copy=True):
         """stream += y * rsqrt(mean(y^2) + eps) * weight, row by row in float32 (y [T, width] of any float
         dtype; None: nothing is added).  Returns the updated stream in the activation dtype, rounded once
@@ -135,19 +178,21 @@ class KernelBackend:
 
     # ---- attention through a cached latent (one shared latent "head" of kv_rank + rot_dim numbers a token)
     def latent_kv_store(self, sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache,
-                        slot_mapping, also_norm=None):
+                        slot_mapping, also_norm=None, layout="interleaved"):
         """Columns [col, col + kv_rank + rot_dim) of ``sums`` [T, *] float32 are a token's down-projection.  The
         first kv_rank, RMS-normed with ``norm_weight``, are its latent c; of the last rot_dim the first
-        2 * len(inv_freq) turn in adjacent pairs (2i, 2i + 1) by the angle position * inv_freq[i] (32-bit).
+        2 * len(inv_freq) turn in adjacent pairs (2i, 2i + 1) (``layout`` "half": pairs (i, i + len(inv_freq))) by the
+        angle position * inv_freq[i] (32-bit).
         Token t's slot of k_cache [pages, 1, page, P] gets [c | turned part | zeros], of v_cache [pages, 1, P, page]
         [c | zeros] (P = the cache's padded size >= kv_rank + rot_dim).  ``also_norm`` = (col, n, weight): the same call
         also returns rmsnorm_columns(sums, col, n, weight, eps) (the query latent beside the key/value latent)."""
         raise NotImplementedError
 
-    def latent_query_rotate_(self, q, num_heads, kv_rank, padded_dim, positions, inv_freq):
+    def latent_query_rotate_(self, q, num_heads, kv_rank, padded_dim, positions, inv_freq, layout="interleaved"):
         """q [T, H padded_dim], every head laid out as the cache's key rows are ([against the latent | rotated part | 0]):
         the first 2 * len(inv_freq) numbers of each head's rotated part (columns kv_rank ..) turn in place in adjacent
-        pairs by the angle position * inv_freq[i].  Returns q."""
+        pairs (``layout`` "half": element i with element i + len(inv_freq)) by the angle position * inv_freq[i].
+        Returns q."""
         raise NotImplementedError
 
     def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):
@@ -179,11 +224,12 @@ class KernelBackend:
         raise NotImplementedError
 
     # ---- routed experts
-    def route_topk(self, logits, bias, top, over="chosen", choice_bias=None):
+    def route_topk(self, logits, bias, top, over="chosen", choice_bias=None, renormalise=False):
         """logits [T, E] float32 (+ bias [E]).  ``over`` "chosen": the ``top`` largest of a token (lowest index first
         among equals), in falling order, and the softmax over those alone.  ``over`` "all": scores = softmax over all
         E; chosen are the ``top`` largest of scores + choice_bias (float32 [E] or None; lowest index first among
-        equals, falling order) and the shares are the chosen ones' scores as they are, not renormalised.
+        equals, falling order) and the shares are the chosen ones' scores as they are, or, with ``renormalise``,
+        divided by their sum + 1e-20.
         -> (experts [T, top] int32, shares [T, top] float32)."""
         raise NotImplementedError
 
@@ -197,10 +243,10 @@ class KernelBackend:
                        glu_block=0):
         """y[t] = sum_j shares[t, j] * W_down[e] act(W_up[e] x[t]), e = experts[t, j]; w_up [E, ff, width],
         w_down [E, width, ff]; the hidden activation is rounded once to the activation dtype -> [T, width] float32.
-        ``gated`` = (limit, alpha): w_up is [E, 2 ff, width], an expert's gate rows before its up rows (or in
-        alternating blocks of ``glu_block`` gate rows and as many up rows: see glu_rows_block), and the hidden
-        activation is g * sigmoid(alpha g) * (u + 1) with g = min(gate sum, limit), u = clamp(up sum, -limit, limit),
-        ``activation`` unused.  ``identity_from`` = E: a choice e >= E is an expert that returns x[t] itself (such
+        ``gated`` = (limit, alpha) or (limit, alpha, shift): w_up is [E, 2 ff, width], an expert's gate rows before its
+        up rows (or in alternating blocks of ``glu_block`` gate rows and as many up rows: see glu_rows_block), and the
+        hidden activation is g * sigmoid(alpha g) * (u + shift) with g = min(gate sum, limit), u = clamp(up sum, -limit,
+        limit), shift 1 unless given (limit infinite, alpha 1, shift 0: silu(gate) * up), ``activation`` unused.  ``identity_from`` = E: a choice e >= E is an expert that returns x[t] itself (such
         choices may be all there are: w_up and w_down None)."""
         raise NotImplementedError
 
@@ -230,10 +276,12 @@ class KernelBackend:
 
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
                    layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None,
-                   norm_per_head=False):
+                   norm_per_head=False, col_bias=None, position_temperature=None):
         """What lies between a q/k/v projection's float32 sums [T, *] and attention, in 32-bit: queries are columns
         [q_col, q_col + Hq dim), keys [k_col, k_col + Hkv dim), values [v_col, v_col + Hkv vdim), or, with ``v_col``
-        None, the keys as projected (vdim = dim).  ``q_norm`` / ``k_norm`` (float32 [Hq dim] / [Hkv dim]): RMS norm over
+        None, the keys as projected (vdim = dim).  ``col_bias`` (float32, one number a column of the sums): the
+        projection's biases, added first.  ``position_temperature`` = (coef, every): the query at position p is
+        multiplied by 1 + coef * ln(floor((p + 1) / every) + 1), every a whole number of positions.  ``q_norm`` / ``k_norm`` (float32 [Hq dim] / [Hkv dim]): RMS norm over
         the whole of a token's queries (keys) at once, times that weight, before anything else; with ``norm_per_head`` the
         norm is taken head by head over the head's dim numbers and the weights are float32 [dim], one for all query
         heads and one for all key heads.  Then the first
@@ -287,8 +335,18 @@ class KernelBackend:
                              v_cache, slot_mapping)
         return qkv
 
+    def gla(self, sums, cols, num_heads, dim, vdim, w_decay, decay_bias, tau, q_scale, norm_weight, eps, state, step):
+        """Gated linear attention from one product's float32 sums [T, *].  ``cols``: first column of q, k (H dim each),
+        of v and the output gate g (H vdim each) and of the decay's inner activations a (w_decay.shape[1] of them).  Per
+        token, head and key channel, in 32-bit: alpha = sigmoid(w_decay a + decay_bias)^(1 / tau).  Per row and head,
+        tokens in order, from the row's slot of ``state`` [slots, H, dim, vdim] float32 (S[i, j]: key channel i, value
+        channel j), left there afterwards: S <- diag(alpha) S + k v^T; o = S^T (q * q_scale).
+        -> rmsnorm(o over a head, eps) * norm_weight [vdim] * silu(g)  [T, H * vdim] in the activation dtype."""
+        raise NotImplementedError
+
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
-                        window, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None):
+                        window, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None,
+                        distance_bias=None):
         """For token t of row r at position p: softmax over keys max(0, p - window + 1)..p
         of row r (read through group.block_tables[r]) of (q . k) * scale, times v.
         q head i uses kv head i // (Hq / Hkv).  q is the first Hq * D columns of
@@ -296,7 +354,9 @@ class KernelBackend:
         denominator, with no value.  ``chunk`` (a number of positions): keys before floor(p / chunk) * chunk are not
         seen either.  ``softcap`` (c > 0): the scaled scores pass through c * tanh(score / c).  ``weights`` "sigmoid":
         no softmax; a visible key counts with sigmoid(score + head_bias[i]) (head_bias float32 [Hq] or None), not
-        normalised over the keys (no sink).  Returns [T, Hq * D] in act_dtype."""
+        normalised over the keys (no sink).  ``distance_bias`` (float32 [Hq, N]): a key n positions back of the query
+        adds distance_bias[i, min(n, N - 1)] to query head i's score, after scale and cap.
+        Returns [T, Hq * D] in act_dtype."""
         raise NotImplementedError
 
     def sample(self, logits, temperatures, seeds, counters, out=None):

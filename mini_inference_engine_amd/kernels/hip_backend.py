@@ -427,6 +427,60 @@ class HipBackend(KernelBackend):
         library.check(lib, lib.mie_scale(_ptr(t), t.numel(), float(factor), self._stream()))
         return t
 
+    def scale_softcap_(self, t, scale, cap):
+        self._on_device(t)
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise ValueError("scale_softcap_: a contiguous float32 tensor")
+        if cap is not None and not cap > 0:
+            raise ValueError(f"scale_softcap_: cap {cap}")
+        lib = self.lib("layer_norm")
+        library.check(lib, lib.mie_scale_softcap(_ptr(t), t.numel(), float(scale), float(cap or 0.0), self._stream()))
+        return t
+
+    def add_layernorm(self, x, residual, weight, bias, eps, out_dtype=None, rows=None):
+        self._on_device(x, residual, weight, bias, rows)
+        out_dtype = out_dtype or self.act_dtype
+        if residual.dtype != torch.float32 or residual.dim() != 2 or not residual.is_contiguous():
+            raise ValueError("add_layernorm: the residual stream must be contiguous float32 [T, width]")
+        T, W = residual.shape
+        if x is not None and (tuple(x.shape) != (T, W) or not x.is_contiguous()):
+            raise ValueError(f"add_layernorm: x {tuple(x.shape)} does not match the stream {(T, W)}")
+        self._f32_vector(weight, W, "add_layernorm: weight")
+        self._f32_vector(bias, W, "add_layernorm: bias")
+        n = T
+        if rows is not None:
+            if rows.dtype != torch.int32 or rows.dim() != 1 or not rows.is_contiguous():
+                raise ValueError("add_layernorm: rows must be contiguous int32")
+            n = rows.shape[0]
+        y = torch.empty((n, W), dtype=out_dtype, device=residual.device)
+        lib = self.lib("layer_norm")
+        library.check(lib, lib.mie_add_layernorm(_ptr(x), _code(x.dtype) if x is not None else F32, _ptr(residual), _ptr(weight),
+                                                 _ptr(bias), _ptr(y), _code(out_dtype), _ptr(rows), n, W, float(eps),
+                                                 self._stream()))
+        return y
+
+    def branch_layernorm_add(self, y, stream, weight, bias, eps, next_norm=None):
+        self._on_device(y, stream, weight, bias)
+        if stream.dtype != torch.float32 or stream.dim() != 2 or not stream.is_contiguous():
+            raise ValueError("branch_layernorm_add: the stream must be contiguous float32 [T, width]")
+        T, W = stream.shape
+        if tuple(y.shape) != (T, W) or not y.is_contiguous():
+            raise ValueError(f"branch_layernorm_add: y {tuple(y.shape)} does not match the stream {(T, W)}")
+        self._f32_vector(weight, W, "branch_layernorm_add: weight")
+        self._f32_vector(bias, W, "branch_layernorm_add: bias")
+        x, nw, nb, ne = None, None, None, 0.0
+        if next_norm is not None:
+            nw, nb, ne = next_norm
+            self._on_device(nw, nb)
+            self._f32_vector(nw, W, "branch_layernorm_add: the next norm's weight")
+            self._f32_vector(nb, W, "branch_layernorm_add: the next norm's bias")
+            x = torch.empty((T, W), dtype=self.act_dtype, device=stream.device)
+        lib = self.lib("layer_norm")
+        library.check(lib, lib.mie_branch_layernorm_add(_ptr(y), _code(y.dtype), _ptr(stream), _ptr(weight), _ptr(bias), float(eps),
+                                                        _ptr(nw), _ptr(nb), float(ne), _ptr(x), _code(self.act_dtype), T, W,
+                                                        self._stream()))
+        return x
+
     def branch_norm_add(self, y, stream, weight, eps, copy=True):
         self._on_device(y, stream, weight)
         if stream.dtype != torch.float32 or stream.dim() != 2 or not stream.is_contiguous():
@@ -510,11 +564,14 @@ class HipBackend(KernelBackend):
         return page, P
 
     def latent_kv_store(self, sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache,
-                        slot_mapping, also_norm=None):
+                        slot_mapping, also_norm=None, layout="interleaved"):
         self._on_device(sums, norm_weight, positions, inv_freq, k_cache, v_cache, slot_mapping)
+        if layout not in self.LAYOUTS:
+            raise ValueError(f"latent_kv_store: layout {layout!r} (interleaved or half)")
         if also_norm is not None and (k_cache.dtype != self.act_dtype or also_norm[2].dtype != norm_weight.dtype):
             # the kernel writes both in one dtype and reads both weights in one: otherwise two calls
-            self.latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slot_mapping)
+            self.latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slot_mapping,
+                                 layout=layout)
             return self.rmsnorm_columns(sums, also_norm[0], also_norm[1], also_norm[2], eps)
         sp = self._f32_columns(sums, col, kv_rank + rot_dim, "latent_kv_store")
         T = sums.shape[0]
@@ -539,11 +596,13 @@ class HipBackend(KernelBackend):
         library.check(lib, lib.mie_latent_kv_store(
             sp, sums.stride(0), _ptr(norm_weight), _code(norm_weight.dtype), float(eps), _ptr(positions), _ptr(inv_freq), n_freq,
             _ptr(k_cache), _ptr(v_cache), _code(k_cache.dtype), _ptr(slot_mapping), T, kv_rank, rot_dim, P, page,
-            qp, qw, _ptr(q_out), qn, self._stream()))
+            qp, qw, _ptr(q_out), qn, self.LAYOUTS[layout], self._stream()))
         return q_out
 
-    def latent_query_rotate_(self, q, num_heads, kv_rank, padded_dim, positions, inv_freq):
+    def latent_query_rotate_(self, q, num_heads, kv_rank, padded_dim, positions, inv_freq, layout="interleaved"):
         self._on_device(q, positions, inv_freq)
+        if layout not in self.LAYOUTS:
+            raise ValueError(f"latent_query_rotate_: layout {layout!r} (interleaved or half)")
         _rows_ok(q, "latent_query_rotate_: q")
         H, P, T = num_heads, padded_dim, q.shape[0]
         n_freq = inv_freq.numel()
@@ -554,7 +613,7 @@ class HipBackend(KernelBackend):
         self._f32_vector(inv_freq, n_freq, "latent_query_rotate_: inv_freq")
         lib = self.lib("latent_attention")
         library.check(lib, lib.mie_latent_query_rotate(_ptr(q), q.stride(0), _code(q.dtype), _ptr(positions), _ptr(inv_freq),
-                                                       n_freq, T, H, kv_rank, P, self._stream()))
+                                                       n_freq, T, H, kv_rank, P, self.LAYOUTS[layout], self._stream()))
         return q
 
     def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):
@@ -645,10 +704,10 @@ class HipBackend(KernelBackend):
         return out
 
     # ---- routed experts
-    def route_topk(self, logits, bias, top, over="chosen", choice_bias=None):
+    def route_topk(self, logits, bias, top, over="chosen", choice_bias=None, renormalise=False):
         self._on_device(logits, bias, choice_bias)
-        if over not in ("chosen", "all") or (choice_bias is not None and over != "all"):
-            raise ValueError(f"route_topk: shares over {over!r} (chosen or all; a choice bias goes with all)")
+        if over not in ("chosen", "all") or ((choice_bias is not None or renormalise) and over != "all"):
+            raise ValueError(f"route_topk: shares over {over!r} (chosen or all; a choice bias or renormalised shares go with all)")
         if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
             raise ValueError("route_topk: logits must be float32 [T, experts] with unit inner stride")
         T, E = logits.shape
@@ -663,7 +722,7 @@ class HipBackend(KernelBackend):
             if choice_bias is not None:
                 self._f32_vector(choice_bias, E, "route_topk: choice bias")
             library.check(lib, lib.mie_route_topk_all(_ptr(logits), logits.stride(0), _ptr(bias), _ptr(choice_bias), _ptr(experts),
-                                                      _ptr(shares), T, E, top, self._stream()))
+                                                      _ptr(shares), T, E, top, int(bool(renormalise)), self._stream()))
             return experts, shares
         library.check(lib, lib.mie_route_topk(_ptr(logits), logits.stride(0), _ptr(bias), _ptr(experts), _ptr(shares), T, E, top,
                                               self._stream()))
@@ -703,6 +762,10 @@ class HipBackend(KernelBackend):
             raise ValueError(f"routed_experts: identity experts from {identity_from} on, but {E} experts have matrices")
         if gated is None and activation not in self.ACT_CODES:
             raise ValueError(f"routed_experts: activation {activation!r}")
+        if gated is not None:
+            gated = (float(gated[0]), float(gated[1]), float(gated[2]) if len(gated) > 2 else 1.0)
+            if not gated[0] > 0:
+                raise ValueError(f"routed_experts: the gate's limit {gated[0]} must be positive (infinite: no clamp)")
         groups = E if identity_from is None else E + 1      # one more group behind the experts holds every identity choice
         offs = torch.empty(groups + 1, dtype=torch.int32, device=dev)
         order = torch.empty(n, dtype=torch.int32, device=dev)
@@ -719,22 +782,22 @@ class HipBackend(KernelBackend):
             # gate and up sums meet in the product's own epilogue: the hidden activation is written once, rounded once
             if self._zeros is None:
                 self._zeros = torch.zeros(64, dtype=torch.int32, device=dev)
-            limit, alpha = gated
+            limit, alpha, shift = gated
             library.check(lib, lib.mie_grouped_glu(_ptr(x), _code(x.dtype), x.stride(0), _ptr(w_up), _code(w_up.dtype), W,
                                                    2 * ff * W, _ptr(hidden), _code(hidden.dtype), ff, _ptr(offs), _ptr(order),
-                                                   top, n, 2 * ff, W, E, float(limit), float(alpha), _ptr(self._zeros),
+                                                   top, n, 2 * ff, W, E, limit, alpha, shift, _ptr(self._zeros),
                                                    self._stream()))
         else:
             if glu_block and ff % glu_block:
                 raise ValueError(f"routed_experts: blocks of {glu_block} rows in experts of inner size {ff}")
-            limit, alpha = gated
+            limit, alpha, shift = gated
             gu = torch.empty((n, 2 * ff), dtype=torch.float32, device=dev)
             self._grouped(x, x.stride(0), 0, 1, w_up, W, 2 * ff * W, gu, 2 * ff, 0, n, 2 * ff, W, E, offs=offs, gather=order,
                           gather_div=top)
             glib = self.lib("gemm")
             # rows of identity choices hold whatever was there: the function of it is never read
             library.check(glib, glib.mie_clamped_glu(_ptr(gu), gu.stride(0), _ptr(hidden), hidden.stride(0), _code(hidden.dtype),
-                                                     n, ff, float(limit), float(alpha), int(glu_block), self._stream()))
+                                                     n, ff, limit, alpha, shift, int(glu_block), self._stream()))
         y = torch.empty((n, W), dtype=torch.float32, device=dev)
         self._grouped(hidden, ff, 0, 1, w_down, ff, W * ff, y, W, 0, n, W, ff, E, offs=offs)
         if identity_from is None:
@@ -829,8 +892,15 @@ class HipBackend(KernelBackend):
 
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
                    layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None,
-                   norm_per_head=False):
-        self._on_device(sums, positions, inv_freq, k_cache, v_cache, slot_mapping, q_norm, k_norm, q_head_scale)
+                   norm_per_head=False, col_bias=None, position_temperature=None):
+        self._on_device(sums, positions, inv_freq, k_cache, v_cache, slot_mapping, q_norm, k_norm, q_head_scale, col_bias)
+        coef, every = 0.0, 0
+        if position_temperature is not None:
+            coef, every = float(position_temperature[0]), int(position_temperature[1])
+            if every < 1 or every != position_temperature[1]:
+                raise ValueError(f"qkv_finish: a query temperature every {position_temperature[1]} positions (a whole number >= 1)")
+        if col_bias is not None:
+            self._f32_vector(col_bias, sums.shape[1], "qkv_finish: col_bias (a number a column of the sums)")
         Hq, Hkv, P, T = num_q_heads, num_kv_heads, padded_dim, sums.shape[0]
         if layout not in self.LAYOUTS:
             raise ValueError(f"qkv_finish: layout {layout!r} (interleaved or half)")
@@ -863,7 +933,8 @@ class HipBackend(KernelBackend):
         library.check(lib, lib.mie_qkv_finish(
             _ptr(sums), sums.stride(0), q_col, k_col, -1 if v_col is None else v_col, _ptr(q_norm), _ptr(k_norm), float(eps),
             int(bool(norm_per_head)), _ptr(inv_freq), nf, self.LAYOUTS[layout], _ptr(q_head_scale), _ptr(positions), _ptr(slot_mapping), _ptr(q),
-            _ptr(k_cache), _ptr(v_cache), _code(self.act_dtype), T, Hq, Hkv, dim, vdim, P, page, self._stream()))
+            _ptr(k_cache), _ptr(v_cache), _code(self.act_dtype), T, Hq, Hkv, dim, vdim, P, page, _ptr(col_bias), coef, every,
+            self._stream()))
         return q
 
     def head_gate_(self, o, gate, gate_col, num_heads, head_dim):
@@ -913,6 +984,47 @@ class HipBackend(KernelBackend):
             _ptr(decay_bias), float(decay_scale), _ptr(removal_bias), _ptr(norm_weight), float(eps), _ptr(state),
             _ptr(step.row_start), _ptr(step.state_slots), _ptr(prep), _ptr(out), _code(out.dtype), T, step.num_rows, H, d,
             chunk, chunks, _ptr(summaries), _ptr(starts), self._stream()))
+        return out
+
+    GLA_CHUNK = 64           # tokens a chunk of the gated linear attention's scan; rows up to this long run whole
+
+    def gla(self, sums, cols, num_heads, dim, vdim, w_decay, decay_bias, tau, q_scale, norm_weight, eps, state, step):
+        self._on_device(sums, w_decay, decay_bias, norm_weight, state)
+        H, d, dv, T = num_heads, dim, vdim, sums.shape[0]
+        if w_decay.dim() != 2 or w_decay.shape[0] != H * d:
+            raise ValueError(f"gla: decay matrix {tuple(w_decay.shape)} for {H} heads of {d}")
+        rank = w_decay.shape[1]
+        self._f32_vector(w_decay, H * d * rank, "gla: decay matrix")
+        for name, n in (("q", H * d), ("k", H * d), ("v", H * dv), ("g", H * dv), ("a", rank)):
+            self._f32_columns(sums, cols[name], n, f"gla: {name}")
+        if decay_bias is not None:
+            self._f32_vector(decay_bias, H * d, "gla: decay_bias")
+        self._f32_vector(norm_weight, dv, "gla: norm_weight")
+        if state.dtype != torch.float32 or tuple(state.shape[1:]) != (H, d, dv) or not state.is_contiguous():
+            raise ValueError(f"gla: state {tuple(state.shape)} for {H} heads of {d} x {dv}")
+        if d > 256 or dv > 256:
+            raise ValueError(f"gla: heads of {d} x {dv} are beyond the 256 x 256 the kernel takes")
+        self._check_rows("gla", step, T)
+        if int(step.host["state_slots"].max()) >= state.shape[0]:
+            raise ValueError("gla: a state slot beyond the state's slots")
+        out = torch.empty((T, H * dv), dtype=self.act_dtype, device=sums.device)
+        decay = torch.empty((T, H * d), dtype=torch.float32, device=sums.device)
+        longest = int(getattr(step, "max_row_tokens", 0) or (step.host["row_start"][1:] - step.host["row_start"][:-1]).max())
+        chunk, chunks, sum_a, sum_b, starts = 0, 0, None, None, None
+        if longest > self.GLA_CHUNK and not self.true_fp32:
+            # rows of many tokens: chunks side by side (whether a step takes this path depends on its longest row alone;
+            # the two paths differ by the rounding of the fold over whole chunks, so the 32-bit mode keeps to one)
+            chunk, chunks = self.GLA_CHUNK, -(-longest // self.GLA_CHUNK)
+            units = step.num_rows * chunks * H
+            sum_a = torch.empty((units, d), dtype=torch.float32, device=sums.device)
+            scratch = torch.empty((2, units, d, dv), dtype=torch.float32, device=sums.device)
+            sum_b, starts = scratch[0], scratch[1]
+        lib = self.lib("gla")
+        library.check(lib, lib.mie_gla(
+            _ptr(sums), sums.stride(0), cols["q"], cols["k"], cols["v"], cols["g"], cols["a"], _ptr(w_decay), rank,
+            _ptr(decay_bias), float(tau), float(q_scale), _ptr(norm_weight), float(eps), _ptr(state), _ptr(step.row_start),
+            _ptr(step.state_slots), _ptr(decay), _ptr(out), _code(out.dtype), T, step.num_rows, H, d, dv, chunk, chunks,
+            _ptr(sum_a), _ptr(sum_b), _ptr(starts), self._stream()))
         return out
 
     def normed_sum_add(self, stream, ys, weights, eps, scale):
@@ -1122,8 +1234,15 @@ class HipBackend(KernelBackend):
 
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
                         window, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None,
-                        force_generic: bool = False, num_splits: int | None = None):
+                        distance_bias=None, force_generic: bool = False, num_splits: int | None = None):
         Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
+        dist_n = 0
+        if distance_bias is not None:
+            self._on_device(distance_bias)
+            if distance_bias.dim() != 2 or distance_bias.shape[0] != Hq or distance_bias.shape[1] < 1:
+                raise ValueError(f"paged_attention: distance_bias {tuple(distance_bias.shape)} for {Hq} query heads")
+            dist_n = distance_bias.shape[1]
+            self._f32_vector(distance_bias, Hq * dist_n, "paged_attention: distance_bias")
         has_sink, sink = int(sink is not None), float(sink or 0.0)
         if weights not in ("softmax", "sigmoid"):
             raise ValueError(f"paged_attention: weights {weights!r} (softmax or sigmoid)")
@@ -1137,7 +1256,7 @@ class HipBackend(KernelBackend):
                 raise ValueError("paged_attention: a bias per head goes with sigmoid weights")
             self._on_device(head_bias)
             self._f32_vector(head_bias, Hq, "paged_attention: head_bias")
-        scored = sigmoid or softcap is not None or chunk is not None
+        scored = sigmoid or softcap is not None or chunk is not None or distance_bias is not None
         if scored and not sigmoid:
             force_generic = True            # a capped or chunked softmax: the 32-bit kernel computes it
         if isinstance(qkv, ProjectionSums):
@@ -1206,7 +1325,7 @@ class HipBackend(KernelBackend):
                     end - done, Hq, Hkv, D, page, float(scale), int(window or 0), has_sink, sink)
             if scored:
                 library.check(lib, lib.mie_paged_attention_scored(*args, int(chunk or 0), float(softcap or 0.0), int(sigmoid),
-                                                                  _ptr(head_bias), self._stream()))
+                                                                  _ptr(head_bias), _ptr(distance_bias), dist_n, self._stream()))
             else:
                 library.check(lib, lib.mie_paged_attention(*args, self._stream()))
         return out

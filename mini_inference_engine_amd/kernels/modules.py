@@ -19,6 +19,11 @@ register_kernel_module("embed_norm", {
     "mie_norm_pair_conv": [P, P, P, P, P, P, P, P, P, P, I, P, I, I, I, I, F, P],
     "mie_branch_norm_conv_single": [P, P, P, F, P, P, P, P, P, I, I, I, I, F, P],
 })
+register_kernel_module("layer_norm", {
+    "mie_add_layernorm": [P, I, P, P, P, P, I, P, I, I, F, P],
+    "mie_branch_layernorm_add": [P, I, P, P, P, F, P, P, F, P, I, I, I, P],
+    "mie_scale_softcap": [P, L, F, F, P],
+})
 register_kernel_module("rope_kv", {
     "mie_rotary_kv_store": [P, I, L, P, P, P, I, I, I, I, P, P, P, I, I, P],
     "mie_rotary_kv_store_sums": [P, L, P, L, P, P, P, P, P, P, I, I, I, I, I, P],
@@ -28,20 +33,20 @@ register_kernel_module("gemm", {
     "mie_silu_mul": [P, L, P, L, I, I, I, P],
     "mie_act_mul": [P, L, P, L, I, I, I, I, P],
     "mie_act_store": [P, L, P, L, I, I, I, I, P],
-    "mie_clamped_glu": [P, L, P, L, I, I, I, F, F, I, P],
+    "mie_clamped_glu": [P, L, P, L, I, I, I, F, F, F, I, P],
 })
 register_kernel_module("grouped_gemm", {
     "mie_grouped_linear": [P, I, L, L, I, P, I, L, L, P, I, L, L, P, P, L, P, P, I, I, I, I, I, I, P, P],
-    "mie_grouped_glu": [P, I, L, P, I, L, L, P, I, L, P, P, I, I, I, I, I, F, F, P, P],
+    "mie_grouped_glu": [P, I, L, P, I, L, L, P, I, L, P, P, I, I, I, I, I, F, F, F, P, P],
     "mie_route_topk": [P, L, P, P, P, I, I, I, P],
-    "mie_route_topk_all": [P, L, P, P, P, P, I, I, I, P],
+    "mie_route_topk_all": [P, L, P, P, P, P, I, I, I, I, P],
     "mie_moe_align": [P, I, I, P, P, P, P],
     "mie_moe_combine": [P, P, P, P, I, I, I, P],
     "mie_moe_combine_identity": [P, P, P, P, I, I, I, P, I, P, I, L, P],
 })
 register_kernel_module("latent_attention", {
-    "mie_latent_kv_store": [P, L, P, I, F, P, P, I, P, P, I, P, I, I, I, I, I, P, P, P, I, P],
-    "mie_latent_query_rotate": [P, L, I, P, P, I, I, I, I, I, P],
+    "mie_latent_kv_store": [P, L, P, I, F, P, P, I, P, P, I, P, I, I, I, I, I, P, P, P, I, I, P],
+    "mie_latent_query_rotate": [P, L, I, P, P, I, I, I, I, I, I, P],
 })
 register_kernel_module("recurrence", {
     "mie_causal_conv": [P, L, P, P, P, P, P, P, P, P, I, I, I, P],
@@ -50,15 +55,18 @@ register_kernel_module("recurrence", {
     "mie_residual_conv": [P, P, P, P, P, P, P, I, I, I, I, I, P],
 })
 register_kernel_module("attention_prep", {
-    "mie_qkv_finish": [P, L, I, I, I, P, P, F, I, P, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+    "mie_qkv_finish": [P, L, I, I, I, P, P, F, I, P, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, F, I, P],
     "mie_head_gate": [P, I, P, L, I, I, I, P],
 })
 register_kernel_module("delta_rule", {
     "mie_delta_rule": [P, L, I, I, I, I, I, I, P, I, P, F, P, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P, P, P],
 })
+register_kernel_module("gla", {
+    "mie_gla": [P, L, I, I, I, I, I, P, I, P, F, F, P, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, P, P],
+})
 register_kernel_module("attention", {
     "mie_paged_attention": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, I, F, P],
-    "mie_paged_attention_scored": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, I, F, I, F, I, P, P],
+    "mie_paged_attention_scored": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, I, F, I, F, I, P, P, I, P],
 })
 register_kernel_module("sampling", {
     "mie_sample": [P, L, P, P, P, P, I, I, P],

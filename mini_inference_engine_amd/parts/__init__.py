@@ -7,8 +7,10 @@ from .block import BranchNormBlock, ParallelBlock, PreNormBlock, SandwichBlock
 from .delta_rule import DeltaRule
 from .dense_ff import DenseFF
 from .embedding import Embedding, LMHead
+from .gla import GatedLinearAttention
 from .input_conv import ConvTail, ResidualConv
 from .latent_attention import LatentAttention, PagedLatent
+from .layernorm import LayerNorm
 from .rglru import RGLRU, RecurrentState
 from .rmsnorm import RMSNorm
 from .rope import NoPosition, RotaryHalfAngles, RotaryHalfSplit, RotaryInterleaved, rotary_tables
@@ -16,4 +18,5 @@ from .routed_experts import RoutedExperts
 from .side_by_side import SideBySide
 from .sigmoid_attention import SigmoidAttention
 from .softmax_attention import SoftmaxAttention
+from .summed_ff import SummedFF
 from .swiglu import SwiGLU

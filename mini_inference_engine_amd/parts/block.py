@@ -41,8 +41,8 @@ class PreNormBlock(Block):
 
 def _sink(residual, norm):
     weight, eps = getattr(norm, "weight", None), getattr(norm, "eps", None)
-    if weight is None or eps is None:
-        return Sink(residual)
+    if weight is None or eps is None or getattr(norm, "kind", "rmsnorm") != "rmsnorm":
+        return Sink(residual)           # a sink names an RMS norm; any other kind is computed by the norm itself
     return Sink(residual, weight, eps)
 
 
@@ -153,7 +153,8 @@ class SandwichBlock(Block):
     stream += norm_mixer_out(mixer(c1(norm_mixer(stream)))); stream += norm_feed_forward_out(feed_forward(c2(
     norm_feed_forward(stream)))).  ``conv_mixer`` / ``conv_feed_forward`` (c1, c2: parts.ResidualConv or None) keep
     their last inputs beside the mixer's cache (CombinedCache members ``mixer``, ``conv1``, ``conv2``).  The
-    feed-forward (with its two norms and its convolution) may be None.  Norms, convolutions and adds are 32-bit;
+    feed-forward (with its two norms and its convolution) may be None.  The norms may be of any kind that has
+    ``add_branch`` (RMS norms, layer norms with weight and bias).  Norms, convolutions and adds are 32-bit;
     the sublayers hand their 32-bit sums to the norm after them.  A sublayer's output is added by whoever reads the
     stream next (kernels.api.NormedBranch): where that is a sublayer with a convolution, one backend call adds the
     normed output and makes the next input."""
@@ -187,11 +188,16 @@ class SandwichBlock(Block):
         ops = self.ops
         if conv is None:
             if pending is not None:
+                return pending.resolve(then=norm)
+            return norm.forward(None, residual)
+        if getattr(norm, "kind", None) != "rmsnorm":     # another kind of norm: in 32-bit, then the convolution
+            if pending is not None:
                 pending.resolve()
-            return ops.add_rmsnorm(None, residual, norm.weight, norm.eps)
+            return conv.forward(norm.forward(None, residual, out_dtype=torch.float32), step, cache.sub(member))
         w = norm.weight if norm.weight.dtype == torch.float32 else norm.weight.float()
         tail = cache.sub(member).tensors["tail"]
-        if pending is not None and pending.y is not None and pending.stream is residual:
+        if (pending is not None and pending.y is not None and pending.stream is residual
+                and getattr(pending.norm, "kind", "rmsnorm") == "rmsnorm"):
             y, pending.y = pending.y, None
             return ops.branch_norm_conv(y, residual, pending.weight, pending.eps, w, norm.eps, conv.weight, tail, step)
         if pending is not None:
@@ -212,9 +218,10 @@ class SandwichBlock(Block):
         combined = self.conv_mixer is not None or self.conv_feed_forward is not None
         x = self._read(pending, residual, self.norm_mixer, self.conv_mixer, cache, "conv1", step)
         a = self.mixer.forward(x, step, cache.sub("mixer") if combined else cache)
-        pending = NormedBranch(ops, a, residual, self.norm_mixer_out.weight, self.norm_mixer_out.eps)
+        pending = NormedBranch(ops, a, residual, self.norm_mixer_out.weight, self.norm_mixer_out.eps, norm=self.norm_mixer_out)
         if self.feed_forward is not None:
             y = self._read(pending, residual, self.norm_feed_forward, self.conv_feed_forward, cache, "conv2", step)
             f = self.feed_forward.forward(y, step)
-            pending = NormedBranch(ops, f, residual, self.norm_feed_forward_out.weight, self.norm_feed_forward_out.eps)
+            pending = NormedBranch(ops, f, residual, self.norm_feed_forward_out.weight, self.norm_feed_forward_out.eps,
+                                   norm=self.norm_feed_forward_out)
         return pending, residual

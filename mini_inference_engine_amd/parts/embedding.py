@@ -2,7 +2,8 @@
 
 stream[t] = E[id[t]] * scale (scale 1 by default), no position term (inference_engine/model.py:96,168);
 logits = y W_lm^T * scale with W_lm = E when tied (inference_engine/model.py:112-113,185; the tied
-table is used as stored, without the embedding's scale).  The stream is 32-bit; logits come out in 32-bit.
+table is used as stored, without the embedding's scale); with ``softcap`` = c the scaled logits pass through
+c * tanh(logits / c).  The stream is 32-bit; logits come out in 32-bit.
 """
 from __future__ import annotations
 
@@ -31,8 +32,11 @@ class Embedding(Part):
 
 class LMHead(Part):
     def __init__(self, vocab_size: int, width: int, weight_name: str, tied_to: Embedding | None = None,
-                 scale: float = 1.0):
+                 scale: float = 1.0, softcap: float | None = None):
         self.scale = float(scale)
+        if softcap is not None and not softcap > 0:
+            raise ValueError("softcap must be positive or None")
+        self.softcap = None if softcap is None else float(softcap)
         self.vocab_size = int(vocab_size)
         self.width = int(width)
         self.weight_name = weight_name
@@ -50,4 +54,6 @@ class LMHead(Part):
 
     def forward(self, y):
         logits = self.ops.linear(y, self.weight, out_dtype=torch.float32)
+        if self.softcap is not None:
+            return self.ops.scale_softcap_(logits, self.scale, self.softcap)
         return logits if self.scale == 1.0 else self.ops.scale_(logits, self.scale)

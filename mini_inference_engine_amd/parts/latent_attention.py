@@ -3,7 +3,9 @@
 Per token the layer keeps c = RMSNorm(W_dkv x)[:kv_rank] and one rotated key part k_r (the last rot_dim
 outputs of W_dkv, position-encoded, shared by all heads).  Head h has key [W_uk,h c | k_r] and value
 W_uv,h c; queries come through a latent of their own, q = W_uq RMSNorm(W_dq x), laid out per head as
-[dim plain | rot_dim rotated].  Score (q_plain . k_plain + q_rot . k_r) * scale, causal, softmax.  The
+[dim plain | rot_dim rotated].  Score (q_plain . k_plain + q_rot . k_r) * scale, causal (with ``window``: over the
+last that many keys only, and pages the window has passed are given back), softmax.  The rotation pairs adjacent
+numbers or the two halves of the turned part, as the position encoding says (``position.layout``).  The
 concatenated heads are multiplied by sigmoid(W_g x) and projected by W_o.
 
 Nothing but c and k_r is cached, and keys are never expanded: q_plain . (W_uk,h c) = (W_uk,h^T q_plain) . c,
@@ -55,13 +57,17 @@ class LatentAttention(Mixer):
 
     def __init__(self, width: int, num_heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, q_rank: int,
                  scale: float, eps: float, position, prefix: str, has_kv: bool = True, gated: bool = True,
-                 tensor_names=None):
+                 tensor_names=None, window: int | None = None):
         self.width, self.num_heads, self.dim, self.rot_dim = int(width), int(num_heads), int(dim), int(rot_dim)
         self.vdim, self.kv_rank, self.q_rank = int(vdim), int(kv_rank), int(q_rank)
         self.scale, self.eps = float(scale), float(eps)
         self.position = position
         self.prefix = prefix
         self.has_kv, self.gated = bool(has_kv), bool(gated)
+        if window is not None and window < 1:
+            raise ValueError("window must be >= 1 or None")
+        self.window = window
+        self.layout = getattr(position, "layout", "interleaved")       # which numbers of the rotated part turn together
         self.names = dict(DEFAULT_NAMES, **(tensor_names or {}))
         if position.rotary_dim > self.rot_dim:
             raise ValueError(f"the position encoding turns {position.rotary_dim} dims; the rotated part has {self.rot_dim}")
@@ -93,7 +99,7 @@ class LatentAttention(Mixer):
         return specs
 
     def cache_requirement(self):
-        return PagedLatent(self.kv_rank, self.rot_dim)
+        return PagedLatent(self.kv_rank, self.rot_dim, self.window)
 
     def prepare(self, device, dtype):
         """Fold W_uk into W_uq (in 32-bit, rounded once to the weights' dtype); the two are not needed afterwards."""
@@ -121,15 +127,16 @@ class LatentAttention(Mixer):
         # one product for everything that reads x: query latent, key/value latent + rotated key part, gate
         sums = ops.linear(x, self.w_down, out_dtype=torch.float32)
         col = self.q_rank
+        half = {} if self.layout == "interleaved" else {"layout": self.layout}
         if self.has_kv:      # the token's cache entry and, in the same kernel, its normed query latent
             cq = ops.latent_kv_store(sums, col, self.kv_rank, self.rot_dim, self.dkv_norm, self.eps, step.positions, inv_freq,
-                                     cache.k, cache.v, group.slot_mapping, also_norm=(0, self.q_rank, self.dq_norm))
+                                     cache.k, cache.v, group.slot_mapping, also_norm=(0, self.q_rank, self.dq_norm), **half)
             col += self.kv_rank + self.rot_dim
         else:
             cq = ops.rmsnorm_columns(sums, 0, self.q_rank, self.dq_norm, self.eps)
         q = ops.latent_query_rotate_(ops.linear(cq, self.w_q), self.num_heads, self.kv_rank, self.padded_dim, step.positions,
-                                     inv_freq)
-        o = ops.paged_attention(q, self.num_heads, 1, self.padded_dim, cache.k, cache.v, group, step, self.scale, None)
+                                     inv_freq, **half)
+        o = ops.paged_attention(q, self.num_heads, 1, self.padded_dim, cache.k, cache.v, group, step, self.scale, self.window)
         heads = ops.latent_value_gate(o, self.w_uv, sums if self.gated else None, col, self.num_heads, self.vdim,
                                       self.kv_rank, self.padded_dim)
         return ops.linear(heads, self.w_o, out_dtype=torch.float32)

@@ -47,3 +47,9 @@ class RMSNorm(Norm):
         if isinstance(x, (Normed, NormedBranch, StreamCopy)):
             return self.lazy(x, residual, rows).materialize(out_dtype)
         return self.ops.add_rmsnorm(x, residual, self.weight, self.eps, out_dtype=out_dtype, rows=rows)
+
+    def add_branch(self, y, stream, then=None):
+        """stream += this norm of y (a sublayer's output).  ``then`` (a Norm): also returns that norm of the updated
+        stream in the activation dtype."""
+        self.ops.branch_norm_add(y, stream, self.weight, self.eps, copy=False)
+        return None if then is None else then.forward(None, stream)

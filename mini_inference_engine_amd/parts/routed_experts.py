@@ -4,10 +4,11 @@ Router logits z = W_r x (+ b_r) in 32-bit.  Two ways from logits to choice and s
   ``shares_over="chosen"``  the ``top`` largest logits are chosen; shares are the softmax over those alone;
   ``shares_over="all"``     scores s = softmax(z) over every router output; chosen are the ``top`` largest of
                             s + c (``choice_bias``: a checkpoint vector c that steers the choice only); shares are the
-                            chosen outputs' s, not renormalised.
+                            chosen outputs' s, not renormalised, or, with ``renormalise``, divided by their sum + 1e-20.
 An expert is W_down act(W_up x) without biases (act: the square of relu unless another of kernels.api.ACTIVATIONS
 is named), or, with ``gated=(limit, alpha)``, W_down (g * sigmoid(alpha g) * (u + 1)) with g = min(W_gate x, limit)
-and u = clamp(W_up x, -limit, limit).  The last ``identity`` router outputs have no tensors: they stand for experts
+and u = clamp(W_up x, -limit, limit); ``gated=(limit, alpha, shift)`` adds ``shift`` to u instead of 1, and
+``gated="silu"`` is the plain gated unit W_down (silu(W_gate x) * W_up x) (no clamp, alpha 1, shift 0).  The last ``identity`` router outputs have no tensors: they stand for experts
 that return x itself.  The output is the share-weighted sum.  The experts' matrices are kept stacked, [experts, ff,
 width] (gate rows before up rows, [experts, 2 ff, width], when gated) and [experts, width, ff], so that one grouped
 product serves all of them.
@@ -21,7 +22,7 @@ from .base import FeedForward, ParamSpec, register_feed_forward
 class RoutedExperts(FeedForward):
     def __init__(self, width: int, inner: int, num_experts: int, top: int, prefix: str, activation: str = "relu2",
                  router_bias: bool = True, tensor_names=None, shares_over: str = "chosen", choice_bias: bool = False,
-                 gated=None, identity: int = 0):
+                 gated=None, identity: int = 0, renormalise: bool = False):
         from ..kernels.api import ACTIVATIONS
         if activation not in ACTIVATIONS:
             raise ValueError(f"activation {activation!r}: one of {ACTIVATIONS}")
@@ -35,7 +36,14 @@ class RoutedExperts(FeedForward):
         self.identity = int(identity)
         self.prefix, self.activation, self.router_bias = prefix, activation, bool(router_bias)
         self.shares_over, self.has_choice_bias = shares_over, bool(choice_bias)
-        self.gated = None if gated is None else (float(gated[0]), float(gated[1]))
+        if renormalise and shares_over != "all":
+            raise ValueError("shares over the chosen outputs alone already sum to one (renormalise goes with shares_over='all')")
+        self.renormalise = bool(renormalise)
+        if gated == "silu":
+            gated = (float("inf"), 1.0, 0.0)
+        self.gated = None if gated is None else tuple(float(g) for g in gated)
+        if self.gated is not None and len(self.gated) not in (2, 3):
+            raise ValueError("gated: (limit, alpha), (limit, alpha, shift) or 'silu'")
         self.names = dict(dict(router="router", router_bias="router.b", expert="e{e}", up="up", down="down", gate="gate",
                                choice_bias="correction"), **(tensor_names or {}))
         self.b_router = self.choice_bias = self.w_up = self.w_down = None
@@ -75,8 +83,12 @@ class RoutedExperts(FeedForward):
         import torch
         ops, E = self.ops, self.num_experts
         logits = ops.linear(x, self.w_router, out_dtype=torch.float32)
-        experts, shares = ops.route_topk(logits, self.b_router if self.router_bias else None, self.top,
-                                         over=self.shares_over, choice_bias=self.choice_bias)
+        if self.renormalise:
+            experts, shares = ops.route_topk(logits, self.b_router if self.router_bias else None, self.top,
+                                             over=self.shares_over, choice_bias=self.choice_bias, renormalise=True)
+        else:
+            experts, shares = ops.route_topk(logits, self.b_router if self.router_bias else None, self.top,
+                                             over=self.shares_over, choice_bias=self.choice_bias)
         rows = self.inner if self.gated is None else 2 * self.inner
         w_up = None if not E else self.w_up.view(E, rows, self.width)
         w_down = None if not E else self.w_down.view(E, self.width, self.inner)

@@ -54,10 +54,11 @@ def ref_turn_pairs(x, positions, inv_freq):
     return out
 
 
-def ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slots):
+def ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slots,
+                        layout="interleaved"):
     P = k_cache.shape[2]
     c = ref_rmsnorm_columns(sums, col, kv_rank, norm_weight, eps, torch.float64)
-    kr = ref_turn_pairs(sums[:, None, col + kv_rank:col + kv_rank + rot_dim].double(), positions, inv_freq)[:, 0]
+    kr = ref_turn(sums[:, None, col + kv_rank:col + kv_rank + rot_dim].double(), positions, inv_freq, layout)[:, 0]
     page, off = slots.long() // P, slots.long() % P
     k_cache[page, 0, off, :] = 0
     k_cache[page, 0, off, :kv_rank] = c.to(k_cache.dtype)
@@ -66,10 +67,10 @@ def ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions
     v_cache[page, 0, :kv_rank, off] = c.to(v_cache.dtype)
 
 
-def ref_latent_query_rotate(q, H, kv_rank, padded, positions, inv_freq):
+def ref_latent_query_rotate(q, H, kv_rank, padded, positions, inv_freq, layout="interleaved"):
     T, n = q.shape[0], 2 * inv_freq.shape[0]
     heads = q.view(T, H, padded)
-    heads[..., kv_rank:kv_rank + n] = ref_turn_pairs(heads[..., kv_rank:kv_rank + n].double(), positions, inv_freq).to(q.dtype)
+    heads[..., kv_rank:kv_rank + n] = ref_turn(heads[..., kv_rank:kv_rank + n].double(), positions, inv_freq, layout).to(q.dtype)
     return q
 
 
@@ -125,21 +126,24 @@ def ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tai
     return out.to(out_dtype)
 
 
-def ref_route_topk(logits, bias, top, over="chosen", choice_bias=None):
+def ref_route_topk(logits, bias, top, over="chosen", choice_bias=None, renormalise=False):
     z = logits.double() if bias is None else logits.double() + bias.double()
     if over == "all":
         scores = torch.softmax(z.float(), -1).double()
         by = scores if choice_bias is None else (scores.float() + choice_bias.float()).double()
         idx = torch.sort(by, dim=-1, descending=True, stable=True).indices[:, :top]
-        return idx.to(torch.int32), torch.gather(scores, 1, idx).float()
+        shares = torch.gather(scores, 1, idx)
+        if renormalise:
+            shares = shares / (shares.sum(-1, keepdim=True) + 1e-20)
+        return idx.to(torch.int32), shares.float()
     order = torch.sort(z, dim=-1, descending=True, stable=True)
     idx, val = order.indices[:, :top], order.values[:, :top]
     return idx.to(torch.int32), torch.softmax(val, -1).float()
 
 
-def ref_clamped_glu(gu, inner, limit, alpha):
+def ref_clamped_glu(gu, inner, limit, alpha, shift=1.0):
     g, u = gu[..., :inner].clamp(max=limit), gu[..., inner:].clamp(min=-limit, max=limit)
-    return g * torch.sigmoid(alpha * g) * (u + 1.0)
+    return g * torch.sigmoid(alpha * g) * (u + shift)
 
 
 def ref_routed_experts(x, experts, shares, w_up, w_down, activation, act_dtype, gated=None, identity_from=None):
@@ -151,7 +155,7 @@ def ref_routed_experts(x, experts, shares, w_up, w_down, activation, act_dtype, 
                 y[t] += shares[t, j].double() * x[t].double()
                 continue
             z = x[t].double() @ w_up[e].double().T
-            h = ref_act(z, activation) if gated is None else ref_clamped_glu(z, z.shape[-1] // 2, gated[0], gated[1])
+            h = ref_act(z, activation) if gated is None else ref_clamped_glu(z, z.shape[-1] // 2, *gated)
             y[t] += shares[t, j].double() * (h.to(act_dtype).double() @ w_down[e].double().T)
     return y.float()
 
@@ -200,7 +204,7 @@ def ref_rotary_kv_store(qkv, positions, cos, sin, rotary_dim, Hq, Hkv, D, k_cach
 
 
 def ref_paged_attention(qkv, Hq, Hkv, D, k_cache, v_cache, block_tables, token_row, positions, scale, window,
-                        out_dtype, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None):
+                        out_dtype, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None, distance_bias=None):
     """Token by token, keys gathered through the block table."""
     T = qkv.shape[0]
     P = k_cache.shape[2]
@@ -222,6 +226,9 @@ def ref_paged_attention(qkv, Hq, Hkv, D, k_cache, v_cache, block_tables, token_r
         s = torch.einsum("hgd,nhd->hgn", q, k) * scale
         if softcap is not None:
             s = softcap * torch.tanh(s / softcap)
+        if distance_bias is not None:
+            n = (p - keys).clamp(max=distance_bias.shape[1] - 1)
+            s = s + distance_bias.double()[:, n].view(Hkv, g, -1)
         if weights == "sigmoid":
             pr = torch.sigmoid(s if head_bias is None else s + head_bias.double().view(Hkv, g, 1))
         elif sink is None:
@@ -265,8 +272,10 @@ def ref_turn(x, positions, inv_freq, layout):
 
 
 def ref_qkv_finish(sums, q_col, k_col, v_col, Hq, Hkv, dim, vdim, P, positions, inv_freq, layout, k_cache, v_cache, slots,
-                   q_norm, k_norm, eps, q_head_scale, out_dtype, norm_per_head=False):
+                   q_norm, k_norm, eps, q_head_scale, out_dtype, norm_per_head=False, col_bias=None, position_temperature=None):
     T = sums.shape[0]
+    if col_bias is not None:
+        sums = (sums.double() + col_bias.double()).float()
     q = sums[:, q_col:q_col + Hq * dim].double()
     k = sums[:, k_col:k_col + Hkv * dim].double()
     v = k if v_col is None else sums[:, v_col:v_col + Hkv * vdim].double()
@@ -282,6 +291,9 @@ def ref_qkv_finish(sums, q_col, k_col, v_col, Hq, Hkv, dim, vdim, P, positions, 
         q, k = ref_turn(q, positions, inv_freq, layout), ref_turn(k, positions, inv_freq, layout)
     if q_head_scale is not None:
         q = q * q_head_scale.double()[None, :, None]
+    if position_temperature is not None:
+        coef, every = position_temperature
+        q = q * (1.0 + coef * torch.log(torch.div(positions.long() + 1, every, rounding_mode="floor").double() + 1.0))[:, None, None]
     page_size = k_cache.shape[2]
     page, off = slots.long() // page_size, slots.long() % page_size
     k_cache[page, :, off, :] = 0
@@ -327,6 +339,58 @@ def ref_normed_sum_add(stream, ys, weights, eps, scale):
         total += yd * torch.rsqrt(yd.pow(2).mean(-1, keepdim=True) + eps) * w.double()
     stream.add_((scale * total).float())
     return stream
+
+
+def ref_layernorm(x, weight, bias, eps):
+    xd = x.double()
+    mean = xd.mean(-1, keepdim=True)
+    var = (xd - mean).pow(2).mean(-1, keepdim=True)
+    return (xd - mean) / torch.sqrt(var + eps) * weight.double() + bias.double()
+
+
+def ref_add_layernorm(x, residual, weight, bias, eps, out_dtype, rows=None):
+    if rows is not None:
+        r = residual[rows.long()].double()
+        if x is not None:
+            r = r + x[rows.long()].double()
+        return ref_layernorm(r, weight, bias, eps).to(out_dtype)
+    if x is not None:
+        residual.add_(x.float())
+    return ref_layernorm(residual, weight, bias, eps).to(out_dtype)
+
+
+def ref_branch_layernorm_add(y, stream, weight, bias, eps, next_norm, act_dtype):
+    stream.add_(ref_layernorm(y, weight, bias, eps).float())
+    if next_norm is None:
+        return None
+    return ref_layernorm(stream, next_norm[0], next_norm[1], next_norm[2]).to(act_dtype)
+
+
+def ref_scale_softcap(t, scale, cap):
+    v = t.double() * scale
+    return (v if cap is None else cap * torch.tanh(v / cap)).float()
+
+
+def ref_gla(sums, cols, H, d, dv, w_decay, decay_bias, tau, q_scale, norm_weight, eps, state, row_start, slots, out_dtype):
+    T = sums.shape[0]
+    x = sums.double()
+    q = x[:, cols["q"]:cols["q"] + H * d].view(T, H, d) * q_scale
+    k = x[:, cols["k"]:cols["k"] + H * d].view(T, H, d)
+    v = x[:, cols["v"]:cols["v"] + H * dv].view(T, H, dv)
+    g = x[:, cols["g"]:cols["g"] + H * dv]
+    z = x[:, cols["a"]:cols["a"] + w_decay.shape[1]] @ w_decay.double().T
+    if decay_bias is not None:
+        z = z + decay_bias.double()
+    alpha = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(T, H, d)
+    out = torch.empty(T, H, dv, dtype=torch.float64, device=sums.device)
+    for row in range(len(slots)):
+        S = state[int(slots[row])].double()
+        for t in range(int(row_start[row]), int(row_start[row + 1])):
+            S = alpha[t][:, :, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            out[t] = torch.einsum("hij,hi->hj", S, q[t])
+        state[int(slots[row])] = S.float()
+    out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.double()
+    return (out.view(T, H * dv) * g * torch.sigmoid(g)).to(out_dtype)
 
 
 def _fmix32(x):
@@ -383,6 +447,22 @@ class TorchBackend(KernelBackend):
     def scale_(self, t, factor):
         return t.mul_(factor)
 
+    def scale_softcap_(self, t, scale, cap):
+        return t.copy_(ref_scale_softcap(t, scale, cap))
+
+    def add_layernorm(self, x, residual, weight, bias, eps, out_dtype=None, rows=None):
+        self._count("add_layernorm")
+        return ref_add_layernorm(x, residual, weight, bias, eps, out_dtype or self.act_dtype, rows)
+
+    def branch_layernorm_add(self, y, stream, weight, bias, eps, next_norm=None):
+        self._count("branch_layernorm_add")
+        return ref_branch_layernorm_add(y, stream, weight, bias, eps, next_norm, self.act_dtype)
+
+    def gla(self, sums, cols, num_heads, dim, vdim, w_decay, decay_bias, tau, q_scale, norm_weight, eps, state, step):
+        self._count("gla")
+        return ref_gla(sums, cols, num_heads, dim, vdim, w_decay, decay_bias, tau, q_scale, norm_weight, eps, state,
+                       step.host["row_start"], step.host["state_slots"], self.act_dtype)
+
     def linear_act(self, x, w, activation="relu2"):
         self._count("linear_act")
         if isinstance(x, Normed):
@@ -404,15 +484,16 @@ class TorchBackend(KernelBackend):
         return (ref_act(gu[:, :intermediate], activation) * gu[:, intermediate:]).to(self.act_dtype)
 
     def latent_kv_store(self, sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache,
-                        slot_mapping, also_norm=None):
+                        slot_mapping, also_norm=None, layout="interleaved"):
         self._count("latent_kv_store")
-        ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slot_mapping)
+        ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slot_mapping,
+                            layout)
         if also_norm is not None:
             return ref_rmsnorm_columns(sums, also_norm[0], also_norm[1], also_norm[2], eps, self.act_dtype)
         return None
 
-    def latent_query_rotate_(self, q, num_heads, kv_rank, padded_dim, positions, inv_freq):
-        return ref_latent_query_rotate(q, num_heads, kv_rank, padded_dim, positions, inv_freq)
+    def latent_query_rotate_(self, q, num_heads, kv_rank, padded_dim, positions, inv_freq, layout="interleaved"):
+        return ref_latent_query_rotate(q, num_heads, kv_rank, padded_dim, positions, inv_freq, layout)
 
     def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):
         return ref_latent_value_gate(o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim, self.act_dtype)
@@ -429,8 +510,8 @@ class TorchBackend(KernelBackend):
         return ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step.host["row_start"],
                               step.host["state_slots"], taps, decay_scale, self.act_dtype)
 
-    def route_topk(self, logits, bias, top, over="chosen", choice_bias=None):
-        return ref_route_topk(logits, bias, top, over, choice_bias)
+    def route_topk(self, logits, bias, top, over="chosen", choice_bias=None, renormalise=False):
+        return ref_route_topk(logits, bias, top, over, choice_bias, renormalise)
 
     def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2", gated=None, identity_from=None, glu_block=0):
         assert glu_block == 0, "the torch operations keep gate rows before up rows"
@@ -467,11 +548,12 @@ class TorchBackend(KernelBackend):
                             k_cache, v_cache, slot_mapping)
 
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
-                        window, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None):
+                        window, sink=None, weights="softmax", softcap=None, chunk=None, head_bias=None, distance_bias=None):
         self._count("paged_attention")
         return ref_paged_attention(qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group.block_tables,
                                    step.token_row, step.positions, scale, window, self.act_dtype, sink=sink,
-                                   weights=weights, softcap=softcap, chunk=chunk, head_bias=head_bias)
+                                   weights=weights, softcap=softcap, chunk=chunk, head_bias=head_bias,
+                                   distance_bias=distance_bias)
 
     def residual_conv(self, h, taps, tail, step, out_dtype=None):
         self._count("residual_conv")
@@ -479,11 +561,11 @@ class TorchBackend(KernelBackend):
 
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
                    layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None,
-                   norm_per_head=False):
+                   norm_per_head=False, col_bias=None, position_temperature=None):
         self._count("qkv_finish")
         return ref_qkv_finish(sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
                               layout, k_cache, v_cache, slot_mapping, q_norm, k_norm, eps, q_head_scale, self.act_dtype,
-                              norm_per_head)
+                              norm_per_head, col_bias, position_temperature)
 
     def head_gate_(self, o, gate, gate_col, num_heads, head_dim):
         o.copy_(ref_head_gate(o, gate, gate_col, num_heads, head_dim))
