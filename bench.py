@@ -3,7 +3,7 @@ Llama-2-7B or Llama-3-8B), random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--shape tinyllama] [--context N] [--layers L]
     python bench.py --kernels [--shape ...] [--batch 8] [--context N]     each dominant kernel alone
-    python bench.py --design zifelorn|vezodra|mutusun [--design-sizes 1024,2048] [--layers R] [--batch 8] [--context 1024]
+    python bench.py --design zifelorn|vezodra|mutusun|labirax [--design-sizes 1024,2048] [--layers R] [--batch 8] [--context 1024]
                                                  that design beside Llama at equal layer sizes (R runs of its layers)
 
 A step is one decode step of the engine (schedule, batch, captured forward, sampling,
@@ -460,10 +460,26 @@ MUTUSUN_SIZES = {
 }
 
 
+# Labirax layer sizes of the same widths: a run of three layers is attention with a distance bias, gated linear attention
+# and latent attention under a window, each with experts (four of them a token, and a shared one: together as large as the
+# dense feed-forward); one more run of the first layer with the same tensors and a cache of its own follows.
+LABIRAX_SIZES = {
+    "1024": dict(vocab=32000, width=1024, heads=16, kv_heads=4, dim=64, latent_heads=8, kv_rank=128, q_rank=384, rot_dim=32,
+                 window=1024, gla_heads=8, gla_dim=64, gla_vdim=128, ff=2816, experts=8, top=3, expert_ff=704, shared_ff=704),
+    "2048": dict(vocab=32000, width=2048, heads=32, kv_heads=8, dim=64, latent_heads=16, kv_rank=192, q_rank=768, rot_dim=64,
+                 window=1024, gla_heads=16, gla_dim=64, gla_vdim=128, ff=5632, experts=16, top=3, expert_ff=1408, shared_ff=1408),
+}
+
+
 def design_configs(design: str, size: str, repeats: int):
     """(the design's configuration, Llama's of the same width, head count, feed-forward size, vocabulary and layer count)."""
-    from mini_inference_engine_amd.config import LlamaConfig, MutusunConfig, VezodraConfig, ZifelornConfig
-    if design == "mutusun":
+    from mini_inference_engine_amd.config import LabiraxConfig, LlamaConfig, MutusunConfig, VezodraConfig, ZifelornConfig
+    if design == "labirax":
+        from mini_inference_engine_amd.models.labirax import _shape
+        z = LABIRAX_SIZES[size]
+        cfg = LabiraxConfig.from_dict(_shape(repeats=repeats, shared=1, **{k: v for k, v in z.items() if k != "ff"}))
+        layers = 3 * repeats + 1
+    elif design == "mutusun":
         from mini_inference_engine_amd.models.mutusun import _shape
         z = MUTUSUN_SIZES[size]
         cfg, layers = MutusunConfig.from_dict(_shape(repeats=repeats, shared=1, **z)), 3 * repeats
@@ -518,7 +534,7 @@ def measure_designs(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["zifelorn", "vezodra", "mutusun"], default=None,
+    ap.add_argument("--design", choices=["zifelorn", "vezodra", "mutusun", "labirax"], default=None,
                     help="instead of the default workload: that design beside Llama at equal layer sizes (decode and prefill)")
     ap.add_argument("--design-sizes", default=None, help="comma-separated widths of --design (default: all of 1024, 2048)")
     ap.add_argument("--gpus", type=int, default=1)

@@ -39,18 +39,22 @@ struct ProjectionSums {
   const int* slots;          // [rows] cache slot of each row's token
 };
 
+// DB: a bias on the softmax's scores by the key's distance, from a table a head (its last entry for everything further
+// back), added after the scale.
 // SIG: sigmoid weights instead of a softmax.  A visible key counts with sigmoid(cap(score) + the head's bias),
 // cap(x) = c tanh(x / c) or x itself; a chunk size n (0: none) hides the keys before floor(position / n) n.  There
 // is no maximum and no denominator: waves and splits simply add up (the merge sees maxima of 0 and one unit sum
 // a workgroup, and the kernel that joins the splits is told not to divide).  scale_log2 then carries the plain scale.
-template <int NW, bool FROM_SUMS, bool SIG = false>
+template <int NW, bool FROM_SUMS, bool SIG = false, bool DB = false>
 __global__ void __launch_bounds__(NW * 64)
 decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache, bf16* v_cache,
                         bf16* __restrict__ out, float* __restrict__ o_part,
                         float* __restrict__ lse_part, const int* __restrict__ block_tables, int max_blocks,
                         const int* __restrict__ positions, int Hq, int Hkv, int head_tiles, int page,
                         float scale_log2, int window, int partition, int num_splits, ProjectionSums proj,
-                        float sink_log2, int chunk, float softcap, const float* __restrict__ head_bias) {
+                        float sink_log2, int chunk, float softcap, const float* __restrict__ head_bias,
+                        const float* __restrict__ dist_bias, int dist_n) {
+  static_assert(!(DB && (SIG || FROM_SUMS)), "the distance bias is built for the softmax over finished queries");
   __shared__ float s_m[NW][16], s_l[NW][16], s_M[16], s_L[16];
   __shared__ float s_o[NW][16][D + 1];
   __shared__ __align__(16) bf16 s_q[FROM_SUMS ? 16 : 1][D];
@@ -157,6 +161,8 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
     }
   }
   int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  // DB: the lane's head's row of the distance table (entries already times log2 e)
+  const float* __restrict__ db_row = DB ? dist_bias + (size_t)head * dist_n : nullptr;
   float sg_c1 = 0.f, sg_c2 = 0.f, sg_c3 = 0.f;
   if constexpr (SIG) {
     if (chunk > 0 && pos / chunk * chunk > lo) lo = pos / chunk * chunk;
@@ -271,7 +277,13 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
       for (int i = 0; i < 4; ++i) {
         const int key = blk + 16 * t + 4 * kb + i;
         ok[t * 4 + i] = key >= lo && key <= pos;
-        sv[t * 4 + i] = ok[t * 4 + i] ? S[t][i] * scale_log2 : -INFINITY;
+        if constexpr (DB) {
+          int n = pos - key;
+          n = n < 0 ? 0 : (n < dist_n ? n : dist_n - 1);            // a key after the row's own is masked
+          sv[t * 4 + i] = ok[t * 4 + i] ? fmaf(S[t][i], scale_log2, db_row[n]) : -INFINITY;
+        } else {
+          sv[t * 4 + i] = ok[t * 4 + i] ? S[t][i] * scale_log2 : -INFINITY;
+        }
         mx = fmaxf(mx, sv[t * 4 + i]);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -450,8 +462,9 @@ static int decode_attention_launch(const void* q, long q_stride, const void* k_c
                                    const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
                                    float scale, int window, int partition, int num_splits, float sink_log2,
                                    hipStream_t stream, bool sigmoid = false, int chunk = 0, float softcap = 0.f,
-                                   const float* head_bias = nullptr) {
+                                   const float* head_bias = nullptr, const float* dist_bias = nullptr, int dist_n = 0) {
   if (rows <= 0) return 0;
+  if (dist_bias && (sigmoid || dist_n < 1)) MIE_FAIL("decode_attention: a distance bias of %d entries a head, softmax only", dist_n);
   if (chunk < 0 || softcap < 0.f) MIE_FAIL("decode_attention: chunk %d, score cap %g", chunk, (double)softcap);
   if (head_dim != D) MIE_FAIL("decode_attention: built for head_dim %d, called with %d", D, head_dim);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("decode_attention: %d query heads on %d kv heads", Hq, Hkv);
@@ -468,24 +481,34 @@ static int decode_attention_launch(const void* q, long q_stride, const void* k_c
   bf16* kc = (bf16*)const_cast<void*>(k_cache);
   bf16* vc = (bf16*)const_cast<void*>(v_cache);
   const bool whole = num_splits == 1 && NW_WHOLE != NW_SPLIT && (long)rows * Hkv * head_tiles < NW_WHOLE_BELOW;
-  if (sigmoid && whole)
+  if (dist_bias && whole)
+    hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, false, false, true>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)q, q_stride,
+                       kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
+                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2, 0, 0.f,
+                       (const float*)nullptr, dist_bias, dist_n);
+  else if (dist_bias)
+    hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, false, false, true>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)q, q_stride,
+                       kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
+                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2, 0, 0.f,
+                       (const float*)nullptr, dist_bias, dist_n);
+  else if (sigmoid && whole)
     hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, false, true>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)q, q_stride,
                        kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
-                       scale, window, partition, num_splits, ProjectionSums{}, sink_log2, chunk, softcap, head_bias);
+                       scale, window, partition, num_splits, ProjectionSums{}, sink_log2, chunk, softcap, head_bias, (const float*)nullptr, 0);
   else if (sigmoid)
     hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, false, true>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)q, q_stride,
                        kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
-                       scale, window, partition, num_splits, ProjectionSums{}, sink_log2, chunk, softcap, head_bias);
+                       scale, window, partition, num_splits, ProjectionSums{}, sink_log2, chunk, softcap, head_bias, (const float*)nullptr, 0);
   else if (whole)
     hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, false>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)q, q_stride,
                        kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
                        scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2, 0, 0.f,
-                       (const float*)nullptr);
+                       (const float*)nullptr, (const float*)nullptr, 0);
   else
     hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, false>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)q, q_stride,
                        kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
                        scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2, 0, 0.f,
-                       (const float*)nullptr);
+                       (const float*)nullptr, (const float*)nullptr, 0);
   MIE_CHECK_LAUNCH("decode_attention");
   if (num_splits > 1) {
     hipLaunchKernelGGL(merge_splits_kernel, dim3(rows * Hq), dim3(64), 0, stream, o_part, lse_part, (bf16*)out, num_splits,
@@ -554,12 +577,12 @@ MIE_EXPORT int mie_decode_attention_from_sums(const float* part, int splits, lon
     hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, true>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)nullptr, 0L,
                        (bf16*)k_cache, (bf16*)v_cache, (bf16*)out, (float*)nullptr, (float*)nullptr, block_tables, max_blocks,
                        positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj, -INFINITY, 0, 0.f,
-                       (const float*)nullptr);
+                       (const float*)nullptr, (const float*)nullptr, 0);
   else
     hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, true>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)nullptr, 0L,
                        (bf16*)k_cache, (bf16*)v_cache, (bf16*)out, (float*)nullptr, (float*)nullptr, block_tables, max_blocks,
                        positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj, -INFINITY, 0, 0.f,
-                       (const float*)nullptr);
+                       (const float*)nullptr, (const float*)nullptr, 0);
   MIE_CHECK_LAUNCH("decode_attention_from_sums");
   return 0;
 }
@@ -623,4 +646,17 @@ MIE_EXPORT int mie_decode_attention_static(const void* q, long q_stride, const v
   float* lse_part = base + entries * D;       // [rows, Hq, splits]
   return mie_decode_attention(q, q_stride, k_cache, v_cache, out, o_part, lse_part, block_tables, max_blocks, positions,
                               rows, Hq, Hkv, head_dim, page, scale, window, partition, num_splits, stream);
+}
+
+// The softmax with a bias on the score by the key's distance: dist_bias float32 [Hq, dist_n], its entries already times
+// log2 e; a key n positions back of the row's token adds entry min(n, dist_n - 1) of the head's row to score * scale.
+MIE_EXPORT int mie_decode_attention_biased(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                           float* o_part, float* lse_part, const int* block_tables, int max_blocks,
+                                           const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
+                                           float scale, int window, int partition, int num_splits, const float* dist_bias,
+                                           int dist_n, hipStream_t stream) {
+  if (!dist_bias) MIE_FAIL("decode_attention_biased: no table");
+  return decode_attention_launch(q, q_stride, k_cache, v_cache, out, o_part, lse_part, block_tables, max_blocks, positions,
+                                 rows, Hq, Hkv, head_dim, page, scale, window, partition, num_splits, -INFINITY, stream, false,
+                                 0, 0.f, nullptr, dist_bias, dist_n);
 }

@@ -32,6 +32,9 @@
 // no denominator, the weights go straight into the second product.  A chunk size n (0: none) hides the keys
 // before floor(position / n) n.  Per score two exponentials and two reciprocals with a cap, one of each without:
 // tanh(y) = 1 - 2 / (1 + 2^(2 y log2 e)), sigmoid(z) = 1 / (1 + 2^(-z log2 e)), the constants folded.
+//
+// DB: a bias on the softmax's scores by the key's distance, from a table a head (its last entry for everything
+// further back), added after the scale; the running maximum then lives in units of log2 e of the biased score.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // Waves a workgroup, at head sizes up to 128 (above, eight waves do not fit the registers: always 4):
@@ -74,14 +77,15 @@ __device__ __forceinline__ float pair_sum(float x) {
 // KS = 2: the waves form two halves that take the even and the odd 64-key blocks of the same queries (a step
 // brings 128 keys in, each half computes its 64) and join their results at the end: half the blocks a wave
 // for rows too short to give every SIMD two waves otherwise.
-template <int PF_WAVES, int KS, bool SIG>
+template <int PF_WAVES, int KS, bool SIG, bool DB = false>
 __global__ void __launch_bounds__(PF_WAVES * 64)
 prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* __restrict__ k_cache,
                          const bf16* __restrict__ v_cache, bf16* __restrict__ out,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ row_start,
                          const int* __restrict__ row_position, int first_row, int Hq, int Hkv, int waves_h,
                          int page, float scale_log2, int window, float sink_log2, int chunk, float softcap,
-                         const float* __restrict__ head_bias) {
+                         const float* __restrict__ head_bias, const float* __restrict__ dist_bias, int dist_n) {
+  static_assert(!(SIG && DB), "the distance bias is built for the softmax");
   extern __shared__ __align__(16) unsigned char pf_lds[];
   constexpr int PF_THREADS = PF_WAVES * 64;
   constexpr int SUB_WAVES = PF_WAVES / KS;                   // waves of one half
@@ -189,6 +193,9 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
     }
     const int blk0 = kmin & ~(PF_BK - 1);
     const int last_blk = kmax & ~(PF_BK - 1);
+    // DB: the head's row of the distance table (its entries already times log2 e); scores leave the bias step scaled
+    const float* __restrict__ db_row = DB ? dist_bias + (size_t)head * dist_n : nullptr;
+    const float sl2 = DB ? 1.f : scale_log2;
 
     float m = -INFINITY, l = 0.f;
     f32x16 O[DT32];
@@ -314,6 +321,33 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
       // every query of the tile sees every key of the block (uniform over the wave)
       const bool whole = blk + PF_BK - 1 <= tile_first && (window <= 0 || blk >= tile_last - window + 1) &&
                          (!SIG || blk >= tile_lo);
+      if constexpr (DB) {
+        // score * scale + table[min(distance, dist_n - 1)], in units of log2 e.  Three cases, each uniform over the wave:
+        // every key of the block beyond the table's reach for every query of the tile (one number for all); every distance
+        // inside the table (a lane's 32 entries lie at fixed offsets from one address); else clamped look-ups.
+        if (tile_ok && tile_first - (blk + PF_BK - 1) >= dist_n - 1) {
+          const float far = db_row[dist_n - 1];
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[u][i] = fmaf(S[u][i], scale_log2, far);
+        } else if (tile_ok && blk + PF_BK - 1 <= tile_first && tile_last - blk <= dist_n - 1) {
+          const float* __restrict__ at = db_row + (qpos - blk) - 4 * g;
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[u][i] = fmaf(S[u][i], scale_log2, at[-(32 * u + 8 * (i >> 2) + (i & 3))]);
+        } else {
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              int n = qpos - (blk + 32 * u + 8 * (i >> 2) + 4 * g + (i & 3));
+              n = n < 0 ? 0 : (n < dist_n ? n : dist_n - 1);          // a key after the query is masked below
+              S[u][i] = fmaf(S[u][i], scale_log2, db_row[n]);
+            }
+        }
+      }
       if constexpr (SIG) {
         if (softcap > 0.f) {
 #pragma unroll
@@ -364,13 +398,13 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
           mx[e] = max3_nn(max3_nn(S[0][4 * e], S[0][4 * e + 1], S[0][4 * e + 2]),
                           max3_nn(S[0][4 * e + 3], S[1][4 * e], S[1][4 * e + 1]), max_nn(S[1][4 * e + 2], S[1][4 * e + 3]));
         const float mxx = pair_max(max_nn(max_nn(mx[0], mx[1]), max_nn(mx[2], mx[3])));
-        const float m_new = max_nn(m, mxx * scale_log2);
+        const float m_new = max_nn(m, mxx * sl2);
         alpha = fast_exp2(m - m_new);
         m = m_new;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) S[u][i] = fast_exp2(fmaf(S[u][i], scale_log2, -m_new));
+          for (int i = 0; i < 16; ++i) S[u][i] = fast_exp2(fmaf(S[u][i], sl2, -m_new));
       } else {
         const int hi = tile_ok ? qpos : -1;                    // a tile that does not exist sees nothing
         const int lo = window > 0 ? hi - window + 1 : 0;
@@ -385,7 +419,7 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
             mx = max_nn(mx, S[u][i]);
           }
         mx = pair_max(mx);
-        const float m_new = max_nn(m, mx * scale_log2);
+        const float m_new = max_nn(m, mx * sl2);
         // a query may see none of this block's keys (it lies before the block, or the block before its window)
         alpha = m_new == -INFINITY ? 1.f : fast_exp2(m - m_new);
         m = m_new;
@@ -393,7 +427,7 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
         for (int u = 0; u < 2; ++u)
 #pragma unroll
           for (int i = 0; i < 16; ++i)
-            S[u][i] = S[u][i] == -INFINITY ? 0.f : fast_exp2(fmaf(S[u][i], scale_log2, -m_new));
+            S[u][i] = S[u][i] == -INFINITY ? 0.f : fast_exp2(fmaf(S[u][i], sl2, -m_new));
       }
       float rs = 0.f;
       Frag pb[4];
@@ -526,8 +560,9 @@ static int prefill_attention_launch(const void* q, long q_stride, const void* k_
                                     const int* row_position, int first_row, int rows, int max_row_tokens, int Hq,
                                     int Hkv, int head_dim, int page, float scale, int window, float sink_log2,
                                     hipStream_t stream, bool sigmoid = false, int chunk = 0, float softcap = 0.f,
-                                    const float* head_bias = nullptr) {
+                                    const float* head_bias = nullptr, const float* dist_bias = nullptr, int dist_n = 0) {
   if (rows <= 0 || max_row_tokens <= 0) return 0;
+  if (dist_bias && (sigmoid || dist_n < 1)) MIE_FAIL("prefill_attention: a distance bias of %d entries a head, softmax only", dist_n);
   if (chunk < 0 || softcap < 0.f) MIE_FAIL("prefill_attention: chunk %d, score cap %g", chunk, (double)softcap);
   if (head_dim != D) MIE_FAIL("prefill_attention: built for head_dim %d, called with %d", D, head_dim);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("prefill_attention: %d query heads on %d kv heads", Hq, Hkv);
@@ -572,9 +607,9 @@ static int prefill_attention_launch(const void* q, long q_stride, const void* k_
   if (grid.y > 65535 || grid.z > 65535) MIE_FAIL("prefill_attention: grid too large (%d rows)", rows);
   const float scale_log2 = sigmoid ? scale : scale * 1.4426950408889634f;      // the sigmoid kernels fold their own constants
   // more LDS than a kernel gets by default is asked for once per kernel and device
-  static bool lds_allowed[6][64] = {};
+  static bool lds_allowed[9][64] = {};
   auto launch = [&](auto kernel, int waves, int lds_bytes) -> int {
-    const int which = kind + (sigmoid ? 3 : 0);
+    const int which = kind + (sigmoid ? 3 : 0) + (dist_bias ? 6 : 0);
     if (lds_bytes > 64 * 1024 && !lds_allowed[which][dev]) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
       if (e != hipSuccess) MIE_FAIL("prefill_attention: %d bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
@@ -582,17 +617,21 @@ static int prefill_attention_launch(const void* q, long q_stride, const void* k_
     }
     hipLaunchKernelGGL(kernel, grid, dim3(waves * 64), lds_bytes, stream, (const bf16*)q, q_stride, (const bf16*)k_cache,
                        (const bf16*)v_cache, (bf16*)out, block_tables, max_blocks, row_start, row_position, first_row, Hq, Hkv,
-                       waves_h, page, scale_log2, window, sink_log2, chunk, softcap, head_bias);
+                       waves_h, page, scale_log2, window, sink_log2, chunk, softcap, head_bias, dist_bias, dist_n);
     return 0;
   };
   int rc = 0;
+  const bool plain = !sigmoid && !dist_bias;
   if constexpr (PF_MAX_WAVES == 8) {
-    if (kind == EIGHT_QUERIES && !sigmoid) rc = launch(prefill_attention_kernel<8, 1, false>, 8, 2 * PF_BUF);
-    if (kind == EIGHT_KEYS && !sigmoid) rc = launch(prefill_attention_kernel<8, 2, false>, 8, 4 * PF_BUF);
+    if (kind == EIGHT_QUERIES && dist_bias) rc = launch(prefill_attention_kernel<8, 1, false, true>, 8, 2 * PF_BUF);
+    if (kind == EIGHT_KEYS && dist_bias) rc = launch(prefill_attention_kernel<8, 2, false, true>, 8, 4 * PF_BUF);
+    if (kind == EIGHT_QUERIES && plain) rc = launch(prefill_attention_kernel<8, 1, false>, 8, 2 * PF_BUF);
+    if (kind == EIGHT_KEYS && plain) rc = launch(prefill_attention_kernel<8, 2, false>, 8, 4 * PF_BUF);
     if (kind == EIGHT_QUERIES && sigmoid) rc = launch(prefill_attention_kernel<8, 1, true>, 8, 2 * PF_BUF);
     if (kind == EIGHT_KEYS && sigmoid) rc = launch(prefill_attention_kernel<8, 2, true>, 8, 4 * PF_BUF);
   }
-  if (kind == FOUR && !sigmoid) rc = launch(prefill_attention_kernel<4, 1, false>, 4, 2 * PF_BUF);
+  if (kind == FOUR && dist_bias) rc = launch(prefill_attention_kernel<4, 1, false, true>, 4, 2 * PF_BUF);
+  if (kind == FOUR && plain) rc = launch(prefill_attention_kernel<4, 1, false>, 4, 2 * PF_BUF);
   if (kind == FOUR && sigmoid) rc = launch(prefill_attention_kernel<4, 1, true>, 4, 2 * PF_BUF);
   if (rc) return rc;
   MIE_CHECK_LAUNCH("prefill_attention");
@@ -629,4 +668,17 @@ MIE_EXPORT int mie_prefill_attention_sigmoid(const void* q, long q_stride, const
   return prefill_attention_launch(q, q_stride, k_cache, v_cache, out, block_tables, max_blocks, row_start, row_position,
                                   first_row, rows, max_row_tokens, Hq, Hkv, head_dim, page, scale, window, -INFINITY, stream,
                                   true, chunk, softcap, head_bias);
+}
+
+// The softmax with a bias on the score by the key's distance: dist_bias float32 [Hq, dist_n], its entries already times
+// log2 e; a key n positions back of the query adds entry min(n, dist_n - 1) of the head's row to score * scale.
+MIE_EXPORT int mie_prefill_attention_biased(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                            const int* block_tables, int max_blocks, const int* row_start,
+                                            const int* row_position, int first_row, int rows, int max_row_tokens, int Hq,
+                                            int Hkv, int head_dim, int page, float scale, int window, const float* dist_bias,
+                                            int dist_n, hipStream_t stream) {
+  if (!dist_bias) MIE_FAIL("prefill_attention_biased: no table");
+  return prefill_attention_launch(q, q_stride, k_cache, v_cache, out, block_tables, max_blocks, row_start, row_position,
+                                  first_row, rows, max_row_tokens, Hq, Hkv, head_dim, page, scale, window, -INFINITY, stream,
+                                  false, 0, 0.f, nullptr, dist_bias, dist_n);
 }

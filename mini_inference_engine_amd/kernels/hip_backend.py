@@ -83,6 +83,7 @@ class HipBackend(KernelBackend):
         self._lt_workspace = None   # device memory the library's product kernels may use
         self._lt_rows = set()       # row counts whose library products get their kernel chosen by timing (prefer_rows)
         self._lt_tuned = set()      # (M, N, K, kind, leading dims) already chosen that way
+        self._log2_tables = {}      # distance-bias tables in units of log2 e, by the address of the table they were made of
         self.true_fp32 = act_dtype == torch.float32
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
 
@@ -1257,8 +1258,17 @@ class HipBackend(KernelBackend):
             self._on_device(head_bias)
             self._f32_vector(head_bias, Hq, "paged_attention: head_bias")
         scored = sigmoid or softcap is not None or chunk is not None or distance_bias is not None
-        if scored and not sigmoid:
+        biased = distance_bias is not None and not sigmoid and softcap is None and chunk is None and not has_sink
+        if scored and not sigmoid and not biased:
             force_generic = True            # a capped or chunked softmax: the 32-bit kernel computes it
+        table2 = None
+        if biased and qkv.dtype == torch.bfloat16 and not force_generic and D <= 256:
+            # the matrix-core kernels work in units of log2 e: the table in those units, made once a table
+            key = distance_bias.data_ptr()
+            held = self._log2_tables.get(key)
+            if held is None or held[0] is not distance_bias:
+                held = self._log2_tables[key] = (distance_bias, (distance_bias * 1.4426950408889634).contiguous())
+            table2 = held[1]
         if isinstance(qkv, ProjectionSums):
             out = self._decode_attention_from_sums(qkv, Hq, Hkv, D, k_cache, v_cache, group, step, scale, window,
                                                    force_generic or num_splits is not None or bool(has_sink))
@@ -1292,6 +1302,8 @@ class HipBackend(KernelBackend):
             if sigmoid:
                 library.check(lib, lib.mie_decode_attention_sigmoid(*args, int(chunk or 0), float(softcap or 0.0),
                                                                     _ptr(head_bias), self._stream()))
+            elif table2 is not None:
+                library.check(lib, lib.mie_decode_attention_biased(*args, _ptr(table2), dist_n, self._stream()))
             elif has_sink:
                 library.check(lib, lib.mie_decode_attention_sink(*args, sink, self._stream()))
             else:
@@ -1311,6 +1323,8 @@ class HipBackend(KernelBackend):
             if sigmoid:
                 library.check(lib, lib.mie_prefill_attention_sigmoid(*args, int(chunk or 0), float(softcap or 0.0),
                                                                      _ptr(head_bias), self._stream()))
+            elif table2 is not None:
+                library.check(lib, lib.mie_prefill_attention_biased(*args, _ptr(table2), dist_n, self._stream()))
             elif has_sink:
                 library.check(lib, lib.mie_prefill_attention_sink(*args, sink, self._stream()))
             else:

@@ -87,6 +87,7 @@ register_kernel_module("attention_bf16", {
     "mie_decode_attention": [P, L, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P],
     "mie_decode_attention_sink": [P, L, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, F, P],
     "mie_decode_attention_sigmoid": [P, L, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, I, F, P, P],
+    "mie_decode_attention_biased": [P, L, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P, I, P],
     "mie_decode_attention_from_sums": [P, I, L, L, P, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, P],
     "mie_decode_attention_static": [P, L, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P],
     "mie_decode_attention_static_setup": [],
@@ -100,6 +101,7 @@ register_kernel_module("prefill_attention_bf16", {
     "mie_prefill_attention": [P, L, P, P, P, P, I, P, P, I, I, I, I, I, I, I, F, I, P],
     "mie_prefill_attention_sink": [P, L, P, P, P, P, I, P, P, I, I, I, I, I, I, I, F, I, F, P],
     "mie_prefill_attention_sigmoid": [P, L, P, P, P, P, I, P, P, I, I, I, I, I, I, I, F, I, I, F, P, P],
+    "mie_prefill_attention_biased": [P, L, P, P, P, P, I, P, P, I, I, I, I, I, I, I, F, I, P, I, P],
 }, variants=_head_variants, flags=["-mllvm", "-amdgpu-mfma-vgpr-form"])
 # lt_gemm: host code only, the engine's own way into the library's matrix products (hipBLASLt) with the choice of
 # kernel per shape kept here.

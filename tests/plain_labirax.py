@@ -70,7 +70,7 @@ def biased_attention(q, k, v, scale, table, farthest):
 
 def attention_mixer(h, W, p, m):
     n = h.shape[0]
-    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m.get("vdim", m["dim"])
     q = (h @ W[f"{p}.q"].T + W[f"{p}.q.b"]).view(n, H, d)
     k = (h @ W[f"{p}.k"].T + W[f"{p}.k.b"]).view(n, G, d)
     v = (h @ W[f"{p}.v"].T + W[f"{p}.v.b"]).view(n, G, dv)
@@ -142,7 +142,7 @@ def gla_scan(q, k, v, alpha, state=None):
 
 def gla_mixer(h, W, p, m, eps):
     n = h.shape[0]
-    H, d, dv = m["heads"], m["dim"], m["vdim"]
+    H, d, dv = m["heads"], m["dim"], m.get("vdim", m["dim"])
     q = (h @ W[f"{p}.q"].T).view(n, H, d) * d ** -0.5
     k = (h @ W[f"{p}.k"].T).view(n, H, d)
     v = (h @ W[f"{p}.v"].T).view(n, H, dv)
@@ -159,11 +159,12 @@ def gated_ff(h, W, p):
 
 def route(h, W, p, top, margins=None):
     """-> (chosen [n, top], weights [n, top]): softmax over all experts, the ``top`` largest, their scores over
-    their sum.  ``margins`` (a list) receives, per token, the gap between the last chosen and the first refused score."""
-    s = torch.softmax(h @ W[f"{p}.router"].T, dim=-1)
+    their sum.  ``margins`` (a list) receives, per token, the gap between the last chosen and the first refused logit."""
+    z = h @ W[f"{p}.router"].T
+    s = torch.softmax(z, dim=-1)
     picked = torch.topk(s, top, dim=-1)
     if margins is not None and top < s.shape[-1]:
-        ranked = torch.sort(s, dim=-1, descending=True).values
+        ranked = torch.sort(z, dim=-1, descending=True).values
         margins += (ranked[:, top - 1] - ranked[:, top]).tolist()
     return picked.indices, picked.values / (picked.values.sum(-1, keepdim=True) + 1e-20)
 
