@@ -38,7 +38,8 @@ def _from_shape(d, key, shapes, tensor, where):
 @dataclass(frozen=True)
 class BiasedAttentionSpec:
     """``temp_coef``, ``temp_every``: the query at position p times 1 + coef * ln(floor((p + 1) / every) + 1);
-    ``buckets`` rows of the distance table, the last one reached at distance ``bias_max`` at the latest."""
+    ``buckets`` rows of the distance table (the first buckets // 2 one distance each), the last one reached at distance
+    ``bias_max`` at the latest."""
     heads: int
     kv_heads: int
     dim: int
@@ -56,17 +57,20 @@ class BiasedAttentionSpec:
         if heads % kv_heads:
             raise ConfigError(f"config.json: {where}heads {heads} is not a multiple of kv_heads {kv_heads}")
         dim = _take_int(d, "dim")
-        temp = _section(d, "q_temp", where)
-        every = temp.get("every")
-        if isinstance(every, float) and every == int(every):
-            every = int(every)
-        if isinstance(every, bool) or not isinstance(every, int) or every < 1:
-            raise ConfigError(f"config.json: {where}q_temp.every must be a whole number of positions >= 1, found {every!r}")
+        coef, every = 0.0, 1               # no q_temp: the query as projected
+        if d.get("q_temp") is not None:
+            temp = _section(d, "q_temp", where)
+            every = temp.get("every")
+            if isinstance(every, float) and every == int(every):
+                every = int(every)
+            if isinstance(every, bool) or not isinstance(every, int) or every < 1:
+                raise ConfigError(f"config.json: {where}q_temp.every must be a whole number of positions >= 1, found {every!r}")
+            coef = _take_float(temp, "coef")
         buckets = _from_shape(d, "buckets", shapes, f"l{owner}.mix.rel", where)
         spec = cls(heads, kv_heads, dim, _take_int(d, "vdim", default=dim), _take_float(d, "scale"),
-                   _take_float(temp, "coef"), every, buckets, _take_float(d, "bias_max"))
-        if buckets < 2 or buckets % 2:
-            raise ConfigError(f"config.json: {where}a distance table of {buckets} rows: an even number >= 2 is computed here")
+                   coef, every, buckets, _take_float(d, "bias_max"))
+        if buckets < 2:
+            raise ConfigError(f"config.json: {where}a distance table of {buckets} rows: at least 2 are computed here")
         if not spec.bias_max > buckets // 2:
             raise ConfigError(f"config.json: {where}bias_max {spec.bias_max} must lie beyond the table's first half ({buckets // 2})")
         return spec

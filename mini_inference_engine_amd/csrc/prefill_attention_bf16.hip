@@ -36,6 +36,7 @@
 // DB: a bias on the softmax's scores by the key's distance, from a table a head (its last entry for everything
 // further back), added after the scale; the running maximum then lives in units of log2 e of the biased score.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+struct __attribute__((packed, aligned(4))) Run4 { float a, b, c, d; };      // four table entries in a row, 4-byte aligned
 
 // Waves a workgroup, at head sizes up to 128 (above, eight waves do not fit the registers: always 4):
 // 8 over twice the queries (twice the queries share each block that is brought in: at head size 128 and 8,192
@@ -306,6 +307,42 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
     auto compute = [&](int set, int blk) {
       const unsigned char* Kb = pf_lds + (set * KS + wk) * PF_BUF + col * PF_KROW + g * 16;
       const unsigned char* Vb = pf_lds + (set * KS + wk) * PF_BUF + PF_KBYTES + col * PF_VROW + g * 16;
+      // DB: the table's entries for this lane's 32 scores, in units of log2 e, asked for before the first product so that
+      // they are there when the scores are: score * scale + table[min(distance, dist_n - 1)].  Three cases, each uniform
+      // over the wave: every key of the block beyond the table's reach for every query of the tile (one number for all);
+      // every distance inside the table (a lane's keys come in runs of four, so its entries do too, falling: one 16-byte
+      // load a run, at any 4-byte address); else clamped look-ups.
+      float tb[DB ? 2 : 1][DB ? 16 : 1];
+      if constexpr (DB) {
+        if (tile_ok && tile_first - (blk + PF_BK - 1) >= dist_n - 1) {
+          const float far = db_row[dist_n - 1];
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) tb[u][i] = far;
+        } else if (tile_ok && blk + PF_BK - 1 <= tile_first && tile_last - blk <= dist_n - 1) {
+          const float* __restrict__ at = db_row + (qpos - blk) - 4 * g;
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const Run4 r = *reinterpret_cast<const Run4*>(at - (32 * u + 8 * e + 3));
+              tb[u][4 * e + 0] = r.d;
+              tb[u][4 * e + 1] = r.c;
+              tb[u][4 * e + 2] = r.b;
+              tb[u][4 * e + 3] = r.a;
+            }
+        } else {
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              int n = qpos - (blk + 32 * u + 8 * (i >> 2) + 4 * g + (i & 3));
+              n = n < 0 ? 0 : (n < dist_n ? n : dist_n - 1);          // a key after the query is masked below
+              tb[u][i] = db_row[n];
+            }
+        }
+      }
       f32x16 S[2];
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
@@ -322,31 +359,10 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
       const bool whole = blk + PF_BK - 1 <= tile_first && (window <= 0 || blk >= tile_last - window + 1) &&
                          (!SIG || blk >= tile_lo);
       if constexpr (DB) {
-        // score * scale + table[min(distance, dist_n - 1)], in units of log2 e.  Three cases, each uniform over the wave:
-        // every key of the block beyond the table's reach for every query of the tile (one number for all); every distance
-        // inside the table (a lane's 32 entries lie at fixed offsets from one address); else clamped look-ups.
-        if (tile_ok && tile_first - (blk + PF_BK - 1) >= dist_n - 1) {
-          const float far = db_row[dist_n - 1];
 #pragma unroll
-          for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) S[u][i] = fmaf(S[u][i], scale_log2, far);
-        } else if (tile_ok && blk + PF_BK - 1 <= tile_first && tile_last - blk <= dist_n - 1) {
-          const float* __restrict__ at = db_row + (qpos - blk) - 4 * g;
-#pragma unroll
-          for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) S[u][i] = fmaf(S[u][i], scale_log2, at[-(32 * u + 8 * (i >> 2) + (i & 3))]);
-        } else {
-#pragma unroll
-          for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              int n = qpos - (blk + 32 * u + 8 * (i >> 2) + 4 * g + (i & 3));
-              n = n < 0 ? 0 : (n < dist_n ? n : dist_n - 1);          // a key after the query is masked below
-              S[u][i] = fmaf(S[u][i], scale_log2, db_row[n]);
-            }
-        }
+          for (int i = 0; i < 16; ++i) S[u][i] = fmaf(S[u][i], scale_log2, tb[u][i]);
       }
       if constexpr (SIG) {
         if (softcap > 0.f) {

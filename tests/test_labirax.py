@@ -224,7 +224,7 @@ def test_config_round_trip_registry_and_sizes_from_tensor_shapes(tmp_path):
     lambda c: c["layers"][0]["mlp"]["router"].update(top=6),               # more than there are experts
     lambda c: c["layers"][0]["mixer"].update(kv_heads=4),                  # 6 query heads over 4 key heads
     lambda c: c["layers"][0]["mixer"].update(bias_max=4),                  # not beyond the table's first half
-    lambda c: c["layers"][0]["mixer"].update(buckets=7),
+    lambda c: c["layers"][0]["mixer"].update(buckets=1),
     lambda c: c["layers"][0]["mixer"]["q_temp"].update(every=0),
     lambda c: c["layers"][0]["mixer"]["q_temp"].update(every=2.5),
     lambda c: c["layers"][1]["mixer"].update(tau=0.0),
