@@ -851,3 +851,51 @@ def test_long_prompts_in_chunks_of_the_recurrence(dtype):
 def test_greedy_generation_through_the_engine(dtype):
     eng = generate("A", "cuda", dtype)
     assert eng.num_graph_steps > 0, "decode steps run as captured graphs"
+
+
+# --------------------------------------------------------------------------------------------- the command line
+def run_cli(*args):
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, "-m", "mini_inference_engine_amd", *args], cwd=root, capture_output=True, text=True,
+                          timeout=600)
+    assert proc.returncode == 0, f"{args}: exit {proc.returncode}\n{proc.stderr[-2000:]}"
+    return proc
+
+
+def test_random_model_of_the_named_size_is_what_the_loader_reads(tmp_path):
+    from safetensors.torch import load_file
+    folder = str(tmp_path / "m")
+    run_cli("random-model", "--shape", "labirax-tiny", "--seed", "3", "--dtype", "float32", "--out", folder)
+    cfg, arch = load_model_config(folder)
+    assert arch.name == "Labirax" and [layer.weights_of for layer in cfg.layers] == [None, None, None, 0, 1]
+    stored = load_file(folder + "/model.safetensors")
+    assert tuple(stored["l0.mix.rel"].shape) == (32, 6) and tuple(stored["l1.mix.a1"].shape) == (16, 64) and "l3.mix.q" not in stored
+    raw = json.loads(open(folder + "/config.json").read())
+    runner = host_runner(cfg, stored, pages=8, rows=2, tokens=64)
+    toks = trace_util.random_prompts(raw["vocab"], [40], seed=1)
+    got = trace_util.run_on_runner(runner, trace_util.portions(toks, sizes=(9, 2, 20)))
+    trace_util.compare(got, expected_logits(raw, stored, toks), F32_TOL, "the named size")
+
+
+@pytest.mark.gpu
+def test_generate_from_the_command_line(tmp_path):
+    from safetensors.torch import load_file
+    folder = str(tmp_path / "m")
+    run_cli("random-model", "--shape", "labirax-tiny", "--seed", "3", "--dtype", "float32", "--out", folder)
+    prompts = [[5, 17, 3, 200, 41], list(range(20, 54)), [7]]
+    args = ["generate", "--model", folder, "--dtype", "float32", "--max-tokens", "6", "--ignore-eos", "--num-blocks", "24", "--quiet"]
+    for p in prompts:
+        args += ["--prompt-ids", ",".join(map(str, p))]
+    lines = [json.loads(line) for line in run_cli(*args).stdout.splitlines() if line.startswith("{")]
+    raw, stored = json.loads(open(folder + "/config.json").read()), load_file(folder + "/model.safetensors")
+    assert [r["prompt_len"] for r in lines] == [len(p) for p in prompts]
+    for prompt, rec in zip(prompts, lines):
+        ids = list(prompt)
+        assert len(rec["output_ids"]) == 6
+        for tok in rec["output_ids"]:
+            row = plain.forward(raw, stored, ids)[-1]
+            assert float(row.max() - row[tok]) <= 1e-5 * float(row.abs().max()), f"token {tok} after {len(ids)} tokens"
+            ids.append(tok)
