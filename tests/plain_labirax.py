@@ -30,10 +30,6 @@ def rms_norm(x, weight, eps):
     return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def silu(z):
     return z * torch.sigmoid(z)
 
