@@ -7,7 +7,7 @@
 //     the logarithm in the form that neither overflows nor cancels (min(z, 0) - log1p(exp(-|z|))).  -> decay [T, H d]
 // gla_scan: a workgroup a (row, chunk, head); thread j owns column j of S in registers (the update of column j reads
 //     that column only), tokens in order.  What all columns share (q * q_scale, k, alpha of a token) comes in through the
-//     LDS, GLA_TB tokens at a time, the next ones already in registers.  The head's output is divided by its root mean
+//     LDS, GLA_TB tokens at a time, the next batch on its way meanwhile.  The head's output is divided by its root mean
 //     square, times the weight and silu of the output gate, and rounded once.
 //
 // Rows run whole (one chunk: S from state[slot], left there afterwards), or, long rows, in chunks of L tokens side by
@@ -87,22 +87,63 @@ gla_scan_kernel(GlaArgs a) {
   for (int i = 0; i < (DK + 63) / 64; ++i) prod[i] = 1.f;
   const int waves = nthreads >> 6, wave = j >> 6, lane = j & 63;
 
+  // What a batch of GLA_TB tokens brings in: q, k and the decays of the head (to the LDS) and this thread's values.  Up to
+  // key sizes of 128 the next batch's numbers are asked for into registers before the current batch is computed (loads
+  // from clamped addresses, never predicated: the compiler would wait for each where it is issued), so that memory's
+  // latency hides behind the recurrence; wider heads have no registers to spare and load where they need.
+  constexpr bool AHEAD = DK <= 128;
+  constexpr int R = AHEAD ? (GLA_TB * DK + 63) / 64 : 1;      // numbers a thread carries when a workgroup is one wave
+  float pq[R], pk[R], pa[R], pv[GLA_TB];
+  auto fetch = [&](int t0) {
+    const int nt = t_end - t0 < GLA_TB ? t_end - t0 : GLA_TB;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      int e = j + r * nthreads;
+      e = e < nt * DK ? e : nt * DK - 1;
+      const int tt = e / DK, i = e - tt * DK, ic = i < d ? i : d - 1;
+      const size_t at = (size_t)(t0 + tt) * a.ld + (size_t)h * d + ic;
+      pq[r] = a.sums[at + a.q_col];
+      pk[r] = a.sums[at + a.k_col];
+      pa[r] = a.decay[((size_t)(t0 + tt) * H + h) * d + ic];
+    }
+#pragma unroll
+    for (int tt = 0; tt < GLA_TB; ++tt)
+      pv[tt] = a.sums[(size_t)(t0 + (tt < nt ? tt : nt - 1)) * a.ld + a.v_col + (size_t)h * dv + (active ? j : 0)];
+  };
+  if (AHEAD && t_begin < t_end) fetch(t_begin);
+
   for (int t0 = t_begin; t0 < t_end; t0 += GLA_TB) {
     const int nt = t_end - t0 < GLA_TB ? t_end - t0 : GLA_TB;
     __syncthreads();
-    for (int e = j; e < nt * DK; e += nthreads) {
-      const int tt = e / DK, i = e - tt * DK;
-      const size_t r = (size_t)(t0 + tt) * a.ld + (size_t)h * d + i;
-      const bool in = i < d;
-      sq[e] = in ? a.sums[r + a.q_col] * a.q_scale : 0.f;
-      sk[e] = in ? a.sums[r + a.k_col] : 0.f;
-      sa[e] = in ? a.decay[((size_t)(t0 + tt) * H + h) * d + i] : 1.f;
-    }
     float v[GLA_TB];
+    if constexpr (AHEAD) {
 #pragma unroll
-    for (int tt = 0; tt < GLA_TB; ++tt)
-      v[tt] = (active && tt < nt) ? a.sums[(size_t)(t0 + tt) * a.ld + a.v_col + (size_t)h * dv + j] : 0.f;
+      for (int r = 0; r < R; ++r) {
+        const int e = j + r * nthreads;
+        if (e < nt * DK) {
+          const bool in = e % DK < d;
+          sq[e] = in ? pq[r] * a.q_scale : 0.f;
+          sk[e] = in ? pk[r] : 0.f;
+          sa[e] = in ? pa[r] : 1.f;
+        }
+      }
+#pragma unroll
+      for (int tt = 0; tt < GLA_TB; ++tt) v[tt] = (active && tt < nt) ? pv[tt] : 0.f;
+    } else {
+      for (int e = j; e < nt * DK; e += nthreads) {
+        const int tt = e / DK, i = e - tt * DK;
+        const size_t r = (size_t)(t0 + tt) * a.ld + (size_t)h * d + i;
+        const bool in = i < d;
+        sq[e] = in ? a.sums[r + a.q_col] * a.q_scale : 0.f;
+        sk[e] = in ? a.sums[r + a.k_col] : 0.f;
+        sa[e] = in ? a.decay[((size_t)(t0 + tt) * H + h) * d + i] : 1.f;
+      }
+#pragma unroll
+      for (int tt = 0; tt < GLA_TB; ++tt)
+        v[tt] = (active && tt < nt) ? a.sums[(size_t)(t0 + tt) * a.ld + a.v_col + (size_t)h * dv + j] : 0.f;
+    }
     __syncthreads();
+    if (AHEAD && t0 + GLA_TB < t_end) fetch(t0 + GLA_TB);          // on its way while this batch is computed
 #pragma unroll
     for (int tt = 0; tt < GLA_TB; ++tt) {
       if (tt < nt) {
