@@ -131,7 +131,7 @@ def prompts_of(n: int, length: int, vocab: int, seed: int):
 
 
 def measure_decode(eng, batch: int, context: int, steps: int, warmup: int, seed: int, vocab: int | None = None):
-    """Median-free, as the contract asks: exactly ``steps`` steps between two synchronisations."""
+    """Median-free: exactly ``steps`` timed steps between two synchronisations."""
     import torch
     from mini_inference_engine_amd import SamplingParams
     # requests whose prompt is in the cache decode while the others' prompts are still being run:
